@@ -1,0 +1,148 @@
+// C-ABI entry points of chunk_gla: argument checks, workspace layout, kernel sequence.
+//
+// forward  (gla.py:483-550):  outer(kv_n, decay_n)  ->  scan(chunk-start states, hidden_final)  ->  out
+// backward (gla.py:552-625):  outer(dstate_n)       ->  reverse scan(d chunk-end states, dhidden_init)
+//                             ->  grad (dq, dk, dv, dlog_fgate)
+#include "gla_chunk_kernels.hpp"
+
+namespace gla {
+
+struct ChunkPlan {
+    int C = 0;       // tokens per workgroup actually used (a divisor of chunk_size)
+    size_t prod = 0, decay = 0, states = 0;   // byte sizes, each rounded up to 256
+};
+
+static size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// The result does not depend on the chunk length (only its rounding does), so chunk sizes above the
+// largest compiled tile run with that tile; sizes below 16 tokens are not built.
+static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, int64_t chunk, int dtype,
+                      ChunkPlan *plan)
+{
+    if (B <= 0 || T <= 0 || H <= 0 || DK <= 0 || DV <= 0) return GLA_ERR_SHAPE;
+    if (B > 65535 || H > 65535 || T > (1 << 30)) return GLA_ERR_SHAPE;
+    if (dtype != GLA_F32 && dtype != GLA_BF16) return GLA_ERR_DTYPE;
+    if (DK != DV) return GLA_ERR_SHAPE;                      // gla.py:499
+    if (!is_pow2(chunk) || T % chunk != 0) return GLA_ERR_CHUNK;   // gla.py:500, 674
+    int64_t C = chunk;
+    const int64_t cmax = dtype == GLA_BF16 ? 128 : 64;
+    if (C > cmax) C = cmax;
+    bool ok = false;
+#define GLA_PLAN_CASE(T_, C_, D_) \
+    if (((dtype == GLA_BF16) == (sizeof(T_) == 2)) && C == C_ && DK == D_) ok = true;
+    GLA_FOR_EACH_CHUNK_CONFIG(GLA_PLAN_CASE)
+#undef GLA_PLAN_CASE
+    if (!ok) return GLA_ERR_UNSUPPORTED;
+    const size_t N = (size_t)(T / C);
+    const size_t esz = dtype == GLA_BF16 ? 2 : 4;
+    plan->C = (int)C;
+    plan->prod = round256((size_t)B * H * N * DK * DV * sizeof(float));
+    plan->decay = round256((size_t)B * H * N * DK * sizeof(float));
+    plan->states = round256((size_t)B * H * N * DK * DV * esz);
+    return GLA_OK;
+}
+
+template <typename F> static int dispatch(int dtype, int C, int D, F &&f)
+{
+#define GLA_DISPATCH_CASE(T_, C_, D_)                                           \
+    if (((dtype == GLA_BF16) == (sizeof(T_) == 2)) && C == C_ && D == D_)       \
+        return f(T_{}, std::integral_constant<int, C_>{}, std::integral_constant<int, D_>{});
+    GLA_FOR_EACH_CHUNK_CONFIG(GLA_DISPATCH_CASE)
+#undef GLA_DISPATCH_CASE
+    return GLA_ERR_UNSUPPORTED;
+}
+
+}  // namespace gla
+
+using namespace gla;
+
+extern "C" size_t gla_chunk_states_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                         int64_t chunk_size, gla_dtype dtype)
+{
+    ChunkPlan p;
+    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.states : 0;
+}
+
+extern "C" size_t gla_chunk_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                                int64_t chunk_size, gla_dtype dtype)
+{
+    ChunkPlan p;
+    // room for the chunk states as well, used when the caller keeps no residual
+    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.prod + p.decay + p.states : 0;
+}
+
+extern "C" size_t gla_chunk_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                                int64_t chunk_size, gla_dtype dtype)
+{
+    ChunkPlan p;
+    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.prod + p.decay + p.states : 0;
+}
+
+extern "C" int gla_chunk_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                             int64_t chunk_size, gla_dtype dtype, const void *hidden_init,
+                             const float *log_fgate, const void *value, const void *key, const void *query,
+                             void *hidden_final, void *out, void *states, void *workspace,
+                             size_t workspace_bytes)
+{
+    ChunkPlan p;
+    int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p);
+    if (rc) return rc;
+    const void *req[] = {hidden_init, log_fgate, value, key, query, hidden_final, out};
+    for (const void *ptr : req) {
+        if (!ptr) return GLA_ERR_NULL;
+        if (!aligned16(ptr)) return GLA_ERR_ALIGN;
+    }
+    if (!workspace || workspace_bytes < p.prod + p.decay + (states ? 0 : p.states)) return GLA_ERR_WORKSPACE;
+    if (!aligned16(workspace) || (states && !aligned16(states))) return GLA_ERR_ALIGN;
+    unsigned char *ws = (unsigned char *)workspace;
+    float *prodT = (float *)ws;
+    float *decay = (float *)(ws + p.prod);
+    void *st_buf = states ? states : (void *)(ws + p.prod + p.decay);
+    hipStream_t st = (hipStream_t)stream;
+    const int N = (int)(T / p.C);
+    return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d) -> int {
+        typedef decltype(t) E;
+        constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value;
+        int e = launch_chunk_outer<E, C_, D_>(st, 0, (int)B, (int)T, (int)H, log_fgate, value, key, prodT, decay);
+        if (e) return e;
+        e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 0, hidden_init, prodT, decay, st_buf, hidden_final);
+        if (e) return e;
+        return launch_chunk_out<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, st_buf, out);
+    });
+}
+
+extern "C" int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                             int64_t chunk_size, gla_dtype dtype, const float *log_fgate, const void *value,
+                             const void *key, const void *query, const void *states,
+                             const void *dhidden_final, const void *dout, void *dhidden_init,
+                             float *dlog_fgate, void *dvalue, void *dkey, void *dquery, void *workspace,
+                             size_t workspace_bytes)
+{
+    ChunkPlan p;
+    int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p);
+    if (rc) return rc;
+    const void *req[] = {log_fgate, value, key, query, states, dhidden_final, dout,
+                         dhidden_init, dlog_fgate, dvalue, dkey, dquery};
+    for (const void *ptr : req) {
+        if (!ptr) return GLA_ERR_NULL;
+        if (!aligned16(ptr)) return GLA_ERR_ALIGN;
+    }
+    if (!workspace || workspace_bytes < p.prod + p.decay + p.states) return GLA_ERR_WORKSPACE;
+    if (!aligned16(workspace)) return GLA_ERR_ALIGN;
+    unsigned char *ws = (unsigned char *)workspace;
+    float *prodT = (float *)ws;
+    float *decay = (float *)(ws + p.prod);
+    void *dstates = (void *)(ws + p.prod + p.decay);
+    hipStream_t st = (hipStream_t)stream;
+    const int N = (int)(T / p.C);
+    return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d) -> int {
+        typedef decltype(t) E;
+        constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value;
+        int e = launch_chunk_outer<E, C_, D_>(st, 1, (int)B, (int)T, (int)H, log_fgate, dout, query, prodT, decay);
+        if (e) return e;
+        e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 1, dhidden_final, prodT, decay, dstates, dhidden_init);
+        if (e) return e;
+        return launch_chunk_grad<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,
+                                            states, dstates, decay, dlog_fgate, dvalue, dkey, dquery);
+    });
+}

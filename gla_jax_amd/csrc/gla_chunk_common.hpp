@@ -1,0 +1,207 @@
+// Building blocks of the chunk_gla kernels (gfx950).
+//
+// Data model.  A workgroup handles one chunk of C tokens of one (batch, head) pair with C/16 waves;
+// wave w owns the 16-token sub-block w.  Inside a wave, lane l = (r, c) with r = l % 16 (token row
+// of the sub-block) and c = l / 16; the lane holds, for its row, the D/4 feature values
+//       d = 32*ks + 8*c + e,   ks = 0..D/32-1, e = 0..7                       ("row layout")
+// which is at the same time the A/B operand layout of the K=32 MFMA when the contraction runs over
+// d (lane (row, c) supplies k-slots 8c..8c+7 of k-step ks).  Products whose output is indexed by
+// (feature, token) are issued as (M = feature, N = token) so that the 4 accumulator rows of a lane
+// are again features of ITS token: with the feature permutation
+//       pi(t, m) = 32*(t/2) + 8*(m/4) + 4*(t%2) + m%4        (t = 16x16 output tile, m = tile row)
+// accumulator element (t, e) of lane (r, c) is feature 32*(t/2) + 8c + 4*(t%2) + e, i.e. element
+// 4t+e of the row layout.  Contractions over tokens read their A operand from natural
+// [token][feature] LDS tiles with the transposing LDS read of gfx950.
+#pragma once
+
+#include "gla_common.hpp"
+
+namespace gla {
+
+struct f32x8 {
+    float v[8];
+};
+
+template <typename T> struct FragTypes;
+template <> struct FragTypes<__bf16> {
+    typedef bf16x8 d8;  // 8 features of one token (one k-step of a feature contraction)
+    typedef bf16x4 t4;  // 4 tokens of one feature (one k-step of a token contraction)
+};
+template <> struct FragTypes<float> {
+    typedef f32x8 d8;
+    typedef f32x4 t4;
+};
+
+// ---- MFMA wrappers ----------------------------------------------------------------------------
+// mma_d: 16x16 += A(16 x 32) B(32 x 16), contraction over 32 features.
+__device__ __forceinline__ f32x4 mma_d(bf16x8 a, bf16x8 b, f32x4 c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mma_d(const f32x8 &a, const f32x8 &b, f32x4 c)
+{
+#pragma unroll
+    for (int e = 0; e < 8; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[e], b.v[e], c, 0, 0, 0);
+    return c;
+}
+// mma_t: 16x16 += A(16 x 16) B(16 x 16), contraction over 16 tokens.
+__device__ __forceinline__ f32x4 mma_t(bf16x4 a, bf16x4 b, f32x4 c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, a),
+                                                     __builtin_bit_cast(short4v, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mma_t(f32x4 a, f32x4 b, f32x4 c)
+{
+#pragma unroll
+    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], c, 0, 0, 0);
+    return c;
+}
+
+// ---- packing ----------------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ typename FragTypes<T>::d8 pack8(const float *x);
+template <> __device__ __forceinline__ bf16x8 pack8<__bf16>(const float *x)
+{
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (__bf16)x[e];
+    return r;
+}
+template <> __device__ __forceinline__ f32x8 pack8<float>(const float *x)
+{
+    f32x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r.v[e] = x[e];
+    return r;
+}
+template <typename T> __device__ __forceinline__ typename FragTypes<T>::t4 pack4(f32x4 x);
+template <> __device__ __forceinline__ bf16x4 pack4<__bf16>(f32x4 x)
+{
+    bf16x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = (__bf16)x[e];
+    return r;
+}
+template <> __device__ __forceinline__ f32x4 pack4<float>(f32x4 x) { return x; }
+
+__device__ __forceinline__ void unpack8(bf16x8 f, float *x)
+{
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = (float)f[e];
+}
+__device__ __forceinline__ void unpack8(const f32x8 &f, float *x)
+{
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = f.v[e];
+}
+
+// ---- memory access ----------------------------------------------------------------------------
+// 8 consecutive features from global or LDS memory (16-byte aligned).
+__device__ __forceinline__ bf16x8 ld8(const __bf16 *p) { return *reinterpret_cast<const bf16x8 *>(p); }
+__device__ __forceinline__ f32x8 ld8(const float *p)
+{
+    f32x4 a = reinterpret_cast<const f32x4 *>(p)[0], b = reinterpret_cast<const f32x4 *>(p)[1];
+    f32x8 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { r.v[e] = a[e]; r.v[4 + e] = b[e]; }
+    return r;
+}
+__device__ __forceinline__ void st8(__bf16 *p, bf16x8 v) { *reinterpret_cast<bf16x8 *>(p) = v; }
+__device__ __forceinline__ void st8(float *p, const f32x8 &v)
+{
+    f32x4 a = {v.v[0], v.v[1], v.v[2], v.v[3]}, b = {v.v[4], v.v[5], v.v[6], v.v[7]};
+    reinterpret_cast<f32x4 *>(p)[0] = a;
+    reinterpret_cast<f32x4 *>(p)[1] = b;
+}
+
+// LDS tiles are row-major [rows][D] with a 16-byte pad per row.
+template <typename T, int D> struct TileGeom {
+    static constexpr int kStride = D + 16 / (int)sizeof(T);
+};
+
+// Transposing LDS read: for a natural [row][col] tile, returns to lane (i = lane % 16) the four
+// elements tile[krow0 + 0..3][colbase(i / 4) + i % 4].  On bf16 this is one ds_read_b64_tr_b16: the
+// 16 lanes of a group each fetch 4 consecutive columns (lane j of the group: row krow0 + j/4,
+// columns colseg .. colseg+3 where colseg is THAT lane's colbase(j % 4)), and the hardware hands lane i
+// column i%4 of the lanes i/4, i/4+4, i/4+8, i/4+12.  `colseg` is therefore colbase(lane%4) and
+// `colown` is colbase((lane%16)/4) + lane%4, both computed by the caller.
+__device__ __forceinline__ bf16x4 lds_tr4(const __bf16 *tile, int stride, int krow0, int colseg, int colown)
+{
+    (void)colown;
+    const int r = threadIdx.x & 15;
+    const __bf16 *p = tile + (krow0 + (r >> 2)) * stride + colseg;
+    typedef __attribute__((ext_vector_type(4))) short v4s;
+    v4s v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)p);
+    return __builtin_bit_cast(bf16x4, v);
+}
+__device__ __forceinline__ f32x4 lds_tr4(const float *tile, int stride, int krow0, int colseg, int colown)
+{
+    (void)colseg;
+    const float *p = tile + krow0 * stride + colown;
+    f32x4 r = {p[0], p[stride], p[2 * stride], p[3 * stride]};
+    return r;
+}
+
+// Column helpers for the feature permutation pi: tile t of a (feature x token) product.
+struct PiCols {
+    int seg, own;
+};
+__device__ __forceinline__ PiCols pi_cols(int t)
+{
+    const int r = threadIdx.x & 15;
+    PiCols p;
+    p.seg = 32 * (t >> 1) + 8 * (r & 3) + 4 * (t & 1);
+    p.own = 32 * (t >> 1) + 8 * (r >> 2) + 4 * (t & 1) + (r & 3);
+    return p;
+}
+// Plain mapping: tile t covers features 16t .. 16t+15, lane i gets feature 16t + i.
+__device__ __forceinline__ PiCols plain_cols(int t)
+{
+    const int r = threadIdx.x & 15;
+    PiCols p;
+    p.seg = 16 * t + 4 * (r & 3);
+    p.own = 16 * t + r;
+    return p;
+}
+
+// ---- gate prefix/suffix hierarchy inside a 16-token sub-block -------------------------------------
+// After `levels` steps (h = 1, 2, 4, ...) p holds the inclusive prefix sum of the gate over the lane's
+// aligned group of size 2h and s the exclusive suffix sum over it; lanes r of a DPP row are the 16
+// tokens.  One step: every lane learns the total of the sibling group and adds it to p (if it sits in
+// the upper sibling) or to s (lower sibling).
+template <int H> __device__ __forceinline__ float sibling_total(float tot)
+{
+    if constexpr (H == 1) return dpp_f32<kDppQuadXor1>(tot);
+    else if constexpr (H == 2) return dpp_f32<kDppQuadXor2>(tot);
+    else if constexpr (H == 4) return dpp_f32<kDppRowHalfMirror>(tot);
+    else return dpp_f32<kDppRowMirror>(tot);
+}
+
+template <int H, int NV> __device__ __forceinline__ void hier_step(float (&p)[NV], float (&s)[NV], bool upper)
+{
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        float other = sibling_total<H>(p[i] + s[i]);
+        p[i] += upper ? other : 0.f;
+        s[i] += upper ? 0.f : other;
+    }
+}
+
+// Sum over the 4 lanes (c = 0..3) that hold the same token row.
+__device__ __forceinline__ float reduce_over_cgroups(float x)
+{
+    x += shfl_xor_f32(x, 16);
+    x += shfl_xor_f32(x, 32);
+    return x;
+}
+
+// Sum over the 16 token rows of the wave (lanes of one DPP row); every lane gets the total.
+__device__ __forceinline__ float reduce_over_rows(float x)
+{
+    x += dpp_f32<kDppQuadXor1>(x);
+    x += dpp_f32<kDppQuadXor2>(x);
+    x += dpp_f32<kDppRowHalfMirror>(x);
+    x += dpp_f32<kDppRowMirror>(x);
+    return x;
+}
+
+}  // namespace gla

@@ -1,0 +1,36 @@
+// Launchers of the chunk_gla kernels, one explicit instantiation per (element type, chunk, head dim).
+#pragma once
+
+#include "gla_common.hpp"
+
+namespace gla {
+
+// (T, C, D) combinations that are compiled.  C = tokens per chunk handled by one workgroup
+// (C/16 waves), D = head dimension (DK == DV, gla.py:499).
+#define GLA_FOR_EACH_CHUNK_CONFIG(M) \
+    M(__bf16, 128, 128)              \
+    M(__bf16, 64, 128)               \
+    M(__bf16, 128, 64)               \
+    M(__bf16, 64, 64)                \
+    M(__bf16, 32, 64)                \
+    M(float, 64, 64)                 \
+    M(float, 32, 64)
+
+template <typename T, int C, int D>
+int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const float *g, const void *x,
+                       const void *y, float *prodT, float *decay);
+
+template <typename T, int D>
+int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hin, const float *prodT,
+                      const float *decay, void *states, void *hout);
+
+template <typename T, int C, int D>
+int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
+                     const void *q, const void *states, void *out);
+
+template <typename T, int C, int D>
+int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
+                      const void *q, const void *dout, const void *states, const void *dstates,
+                      const float *decay, float *dg, void *dv, void *dk, void *dq);
+
+}  // namespace gla

@@ -1,0 +1,210 @@
+// Inter-chunk state path of chunk_gla (gla.py:695-729 forward, gla.py:731-790 backward):
+//
+//   chunk_outer_kernel   per chunk n:  P_n^T[dv][dk] = sum_j X[j][dv] * Y~[j][dk]     (bf16 MFMA, fp32 out)
+//        forward:  X = value, Y~ = key   * exp(L_end - L_j)   -> kv_n      (gla.py:705-708)
+//        backward: X = dout,  Y~ = query * exp(L_j)           -> dstate_n  (gla.py:748-750)
+//     and the chunk decay exp(L_end) per feature.
+//   chunk_scan_kernel    over chunks:  S_{n+1} = decay_n * S_n + P_n  (ops.py:286-297 combine op), written
+//     as the chunk-START states the output kernel needs (gla.py:720-723); run backwards it is the
+//     reverse scan of gla.py:759-765 and yields the gradient w.r.t. every chunk-END state.
+//
+// L is the within-chunk inclusive cumsum of log_fgate (gla.py:509), never written to memory: each
+// wave scans its 16 tokens across lanes, block totals go through a small LDS table.
+// States are kept transposed, [dv][dk], because they are consumed as the A operand of
+// (feature x token) products contracting over dk.
+#include "gla_chunk_common.hpp"
+#include "gla_chunk_kernels.hpp"
+
+namespace gla {
+
+template <typename T, int C, int D, int MODE>
+__global__ __launch_bounds__(C * 4) void chunk_outer_kernel(const float *__restrict__ g,
+                                                            const T *__restrict__ x,
+                                                            const T *__restrict__ y,
+                                                            float *__restrict__ prodT,
+                                                            float *__restrict__ decay, int T_len, int H)
+{
+    constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16;
+    constexpr int LS = TileGeom<T, D>::kStride;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *Xn = reinterpret_cast<T *>(smem);
+    T *Yn = Xn + C * LS;
+    float *rtab = reinterpret_cast<float *>(Yn + C * LS);   // [NB][D]
+
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int r = lane & 15, c = lane >> 4;
+    const int n = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int N = T_len / C;
+    const int64_t tok = (int64_t)b * T_len + (int64_t)n * C + 16 * w + r;
+    const int64_t rowoff = (tok * H + h) * D;
+
+    float p[NV], s[NV];
+    typename FragTypes<T>::d8 yf[KS], xf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = 32 * ks + 8 * c;
+        f32x8 gg = ld8(g + rowoff + d0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
+        yf[ks] = ld8(y + rowoff + d0);
+        xf[ks] = ld8(x + rowoff + d0);
+    }
+    hier_step<1>(p, s, (r & 1) != 0);
+    hier_step<2>(p, s, (r & 2) != 0);
+    hier_step<4>(p, s, (r & 4) != 0);
+    hier_step<8>(p, s, (r & 8) != 0);
+    if (r == 0) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            f32x8 t;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p[8 * ks + e] + s[8 * ks + e]);
+            st8(rtab + w * D + 32 * ks + 8 * c, t);
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) st8(Xn + (16 * w + r) * LS + 32 * ks + 8 * c, xf[ks]);
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = 32 * ks + 8 * c;
+        float f[8], yv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = fast_exp2(MODE == 0 ? s[8 * ks + e] : p[8 * ks + e]);
+        float all[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) all[e] = 1.f;
+        for (int m = 0; m < NB; ++m) {
+            f32x8 t = ld8(rtab + m * D + d0);
+            const bool use = MODE == 0 ? (m > w) : (m < w);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                f[e] *= use ? t.v[e] : 1.f;
+                all[e] *= t.v[e];
+            }
+        }
+        unpack8(yf[ks], yv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) yv[e] *= f[e];
+        st8(Yn + (16 * w + r) * LS + d0, pack8<T>(yv));
+        if (w == 0 && r == 0) {
+            f32x8 t;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) t.v[e] = all[e];
+            st8(decay + (((int64_t)b * H + h) * N + n) * D + d0, t);
+        }
+    }
+    __syncthreads();
+
+    float *outp = prodT + (((int64_t)b * H + h) * N + n) * D * D;
+    for (int mt = w; mt < NT; mt += NB) {
+        f32x4 acc[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const PiCols ca = plain_cols(mt);
+#pragma unroll 2
+        for (int J = 0; J < NB; ++J) {
+            auto a = lds_tr4(Xn, LS, 16 * J + 4 * c, ca.seg, ca.own);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const PiCols cb = plain_cols(nt);
+                auto bb = lds_tr4(Yn, LS, 16 * J + 4 * c, cb.seg, cb.own);
+                acc[nt] = mma_t(a, bb, acc[nt]);
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) outp[(16 * mt + 4 * c + e) * D + 16 * nt + r] = acc[nt][e];
+    }
+}
+
+// One thread = one dv row x 4 consecutive dk of the transposed state.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ hin,
+                                                         const float *__restrict__ prodT,
+                                                         const float *__restrict__ decay,
+                                                         T *__restrict__ states, T *__restrict__ hout,
+                                                         int N, int reverse)
+{
+    const int idx = blockIdx.x * 256 + threadIdx.x;   // over D * D/4
+    const int bh = blockIdx.y;
+    const int dv = idx / (D / 4), dk0 = (idx % (D / 4)) * 4;
+    float X[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) X[e] = Elem<T>::load(hin + (int64_t)bh * D * D + (dk0 + e) * D + dv);
+    const float *pp = prodT + (int64_t)bh * N * D * D + dv * D + dk0;
+    const float *dp = decay + (int64_t)bh * N * D + dk0;
+    T *sp = states + (int64_t)bh * N * D * D + dv * D + dk0;
+    constexpr int U = 4;
+    int step = 0;
+    for (; step + U <= N; step += U) {
+        f32x4 pv[U], dv4[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int n = reverse ? N - 1 - (step + u) : step + u;
+            pv[u] = *reinterpret_cast<const f32x4 *>(pp + (int64_t)n * D * D);
+            dv4[u] = *reinterpret_cast<const f32x4 *>(dp + (int64_t)n * D);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int n = reverse ? N - 1 - (step + u) : step + u;
+            store_vec<T, 4>(sp + (int64_t)n * D * D, X);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) X[e] = dv4[u][e] * X[e] + pv[u][e];
+        }
+    }
+    for (; step < N; ++step) {
+        const int n = reverse ? N - 1 - step : step;
+        f32x4 pv = *reinterpret_cast<const f32x4 *>(pp + (int64_t)n * D * D);
+        f32x4 dd = *reinterpret_cast<const f32x4 *>(dp + (int64_t)n * D);
+        store_vec<T, 4>(sp + (int64_t)n * D * D, X);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) X[e] = dd[e] * X[e] + pv[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) Elem<T>::store(hout + (int64_t)bh * D * D + (dk0 + e) * D + dv, X[e]);
+}
+
+template <typename T, int C, int D>
+int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const float *g, const void *x,
+                       const void *y, float *prodT, float *decay)
+{
+    constexpr int LS = TileGeom<T, D>::kStride;
+    const size_t lds = (size_t)2 * C * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
+    dim3 grid(T_len / C, H, B), block(C * 4);
+    if (mode == 0) {
+        auto kern = chunk_outer_kernel<T, C, D, 0>;
+        if (int e = allow_lds((const void *)kern, lds)) return e;
+        hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)x, (const T *)y, prodT, decay, T_len, H);
+    } else {
+        auto kern = chunk_outer_kernel<T, C, D, 1>;
+        if (int e = allow_lds((const void *)kern, lds)) return e;
+        hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)x, (const T *)y, prodT, decay, T_len, H);
+    }
+    return launch_status();
+}
+
+template <typename T, int D>
+int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hin, const float *prodT,
+                      const float *decay, void *states, void *hout)
+{
+    dim3 grid(D * D / 4 / 256, BH), block(256);
+    hipLaunchKernelGGL((chunk_scan_kernel<T, D>), grid, block, 0, st, (const T *)hin, prodT, decay,
+                       (T *)states, (T *)hout, N, reverse);
+    return launch_status();
+}
+
+#define GLA_INST_OUTER(T, C, D)                                                                       \
+    template int launch_chunk_outer<T, C, D>(hipStream_t, int, int, int, int, const float *, const void *, \
+                                             const void *, float *, float *);
+#define GLA_INST_SCAN(T, D)                                                                           \
+    template int launch_chunk_scan<T, D>(hipStream_t, int, int, int, const void *, const float *,     \
+                                         const float *, void *, void *);
+GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUTER)
+GLA_INST_SCAN(__bf16, 64)
+GLA_INST_SCAN(__bf16, 128)
+GLA_INST_SCAN(float, 64)
+GLA_INST_SCAN(float, 128)
+
+}  // namespace gla

@@ -1,0 +1,148 @@
+// Shared device/host helpers for the gfx950 GLA kernels: element types, MFMA and DPP wrappers,
+// status codes.  Everything here is written for CDNA4 (64-wide wavefronts) only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <type_traits>
+
+#include "../../include/gla_hip.h"
+
+namespace gla {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) short short4v;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---- element traits ---------------------------------------------------------------------------
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static __device__ __forceinline__ float load(const float *p) { return *p; }
+    static __device__ __forceinline__ void store(float *p, float v) { *p = v; }
+};
+template <> struct Elem<__bf16> {
+    static __device__ __forceinline__ float load(const __bf16 *p) { return (float)*p; }
+    static __device__ __forceinline__ void store(__bf16 *p, float v) { *p = (__bf16)v; }
+};
+
+// Loads N consecutive elements (N*sizeof(T) a multiple of 4 and the address aligned to it, up to
+// 16 bytes per access) and widens them to float.
+template <typename T, int N>
+__device__ __forceinline__ void load_vec(const T *p, float (&dst)[N])
+{
+    if constexpr (sizeof(T) == 4) {
+        if constexpr (N % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 4) {
+                f32x4 t = *reinterpret_cast<const f32x4 *>(p + i);
+                dst[i] = t[0]; dst[i + 1] = t[1]; dst[i + 2] = t[2]; dst[i + 3] = t[3];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < N; ++i) dst[i] = p[i];
+        }
+    } else {
+        if constexpr (N % 8 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 8) {
+                bf16x8 t = *reinterpret_cast<const bf16x8 *>(p + i);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) dst[i + j] = (float)t[j];
+            }
+        } else if constexpr (N % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 4) {
+                bf16x4 t = *reinterpret_cast<const bf16x4 *>(p + i);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) dst[i + j] = (float)t[j];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < N; ++i) dst[i] = (float)p[i];
+        }
+    }
+}
+
+template <typename T, int N>
+__device__ __forceinline__ void store_vec(T *p, const float (&src)[N])
+{
+    if constexpr (sizeof(T) == 4) {
+        if constexpr (N % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 4) {
+                f32x4 t = {src[i], src[i + 1], src[i + 2], src[i + 3]};
+                *reinterpret_cast<f32x4 *>(p + i) = t;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < N; ++i) p[i] = src[i];
+        }
+    } else {
+        if constexpr (N % 8 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 8) {
+                bf16x8 t;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) t[j] = (__bf16)src[i + j];
+                *reinterpret_cast<bf16x8 *>(p + i) = t;
+            }
+        } else if constexpr (N % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 4) {
+                bf16x4 t;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) t[j] = (__bf16)src[i + j];
+                *reinterpret_cast<bf16x4 *>(p + i) = t;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < N; ++i) p[i] = (__bf16)src[i];
+        }
+    }
+}
+
+// ---- cross-lane ---------------------------------------------------------------------------------
+// DPP controls (GFX9/CDNA encoding).
+constexpr int kDppQuadXor1 = 0xB1;        // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;        // quad_perm:[2,3,0,1]
+constexpr int kDppRowMirror = 0x140;      // lane r -> 15-r inside a 16-lane row
+constexpr int kDppRowHalfMirror = 0x141;  // lane r -> 7-r inside an 8-lane half row
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+__device__ __forceinline__ float shfl_xor_f32(float v, int mask)
+{
+    return __shfl_xor(v, mask, 64);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---- host side ------------------------------------------------------------------------------
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
+
+// Dynamic LDS above 64 KB has to be granted per kernel before the launch (gfx950 has 160 KB per CU).
+inline int allow_lds(const void *kernel, size_t bytes)
+{
+    if (bytes <= 65536) return 0;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    return e == hipSuccess ? 0 : (int)e;
+}
+
+inline int launch_status()
+{
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int)e;
+}
+
+}  // namespace gla

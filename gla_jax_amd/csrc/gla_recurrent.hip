@@ -1,0 +1,504 @@
+// recurrent_gla forward and backward for gfx950: the per-timestep rank-1 state update
+//   S_t = exp(g_t)[:,None] * S_{t-1} + k_t v_t^T ,   o_t = S_t^T q_t            (gla.py:35-37, 50-96)
+// and its two-sweep gradient (gla.py:271-360, 263).  The [DK,DV] state of one (batch, head) pair
+// lives in the registers of one workgroup for the whole sequence; nothing but inputs, outputs and
+// the final state touches HBM.  fp32 VALU work throughout (the state is fp32, gla.py:89).
+//
+// Register tiling: a wave owns 16 columns (forward) or 16 rows (backward) of the state; a lane owns
+// a 4-wide strip of that and 1/16 of the other dimension, so per step it needs 4 + R inputs per
+// operand, does 3*4*R FMAs and its partial sums are reduced over 16 lanes by xor-shuffles.
+#include "gla_common.hpp"
+
+namespace gla {
+
+// N consecutive elements kept in their memory format until used (halves register use for bf16).
+template <typename T, int N> struct RawVec;
+template <int N> struct RawVec<float, N> {
+    float v[N];
+    __device__ __forceinline__ void load(const float *p) { load_vec<float, N>(p, v); }
+    __device__ __forceinline__ float get(int i) const { return v[i]; }
+};
+template <int N> struct RawVec<__bf16, N> {
+    static constexpr int W = (N + 1) / 2;
+    uint32_t v[W];
+    __device__ __forceinline__ void load(const __bf16 *p)
+    {
+        if constexpr (N == 1) {
+            v[0] = *reinterpret_cast<const uint16_t *>(p);
+        } else if constexpr (N % 8 == 0) {
+#pragma unroll
+            for (int i = 0; i < W; i += 4) {
+                uint4 t = *reinterpret_cast<const uint4 *>(p + 2 * i);
+                v[i] = t.x; v[i + 1] = t.y; v[i + 2] = t.z; v[i + 3] = t.w;
+            }
+        } else if constexpr (N % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < W; i += 2) {
+                uint2 t = *reinterpret_cast<const uint2 *>(p + 2 * i);
+                v[i] = t.x; v[i + 1] = t.y;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < W; ++i) v[i] = *reinterpret_cast<const uint32_t *>(p + 2 * i);
+        }
+    }
+    __device__ __forceinline__ float get(int i) const
+    {
+        uint32_t w = v[i >> 1];
+        return __uint_as_float((i & 1) ? (w & 0xFFFF0000u) : (w << 16));
+    }
+};
+
+// Sum over the 16 lanes that share (lane & 3).
+__device__ __forceinline__ float reduce_over_c(float x)
+{
+    x += shfl_xor_f32(x, 4);
+    x += shfl_xor_f32(x, 8);
+    x += shfl_xor_f32(x, 16);
+    x += shfl_xor_f32(x, 32);
+    return x;
+}
+// Sum over the 4 lanes that share (lane >> 2).
+__device__ __forceinline__ float reduce_over_a(float x)
+{
+    x += dpp_f32<kDppQuadXor1>(x);
+    x += dpp_f32<kDppQuadXor2>(x);
+    return x;
+}
+
+// ------------------------------------------------------------------------------------------------
+// forward.  Block = DV/16 waves = one (b,h); wave w owns state columns [16w, 16w+16); lane (a = l&3,
+// c = l>>2) owns rows [c*RK, (c+1)*RK) x columns 16w + [4a, 4a+4).
+// ------------------------------------------------------------------------------------------------
+template <typename T, typename TO, int RK, int U>
+__global__ __launch_bounds__(RK * 64) void recurrent_fwd_kernel(
+    const T *__restrict__ h0, const float *__restrict__ g, const T *__restrict__ v,
+    const T *__restrict__ k, const T *__restrict__ q, T *__restrict__ hT, TO *__restrict__ out,
+    int T_len, int H, int reverse)
+{
+    constexpr int DK = RK * 16, DV = DK;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int a = lane & 3, c = lane >> 2;
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int dk0 = c * RK, dv0 = wave * 16 + a * 4;
+    const int64_t bh = (int64_t)b * H + h;
+
+    float S[RK][4];
+    {
+        const T *hp = h0 + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+#pragma unroll
+        for (int i = 0; i < RK; ++i) load_vec<T, 4>(hp + (int64_t)i * DV, S[i]);
+    }
+    const int64_t strideK = (int64_t)H * DK, strideV = (int64_t)H * DV;
+    const float *gp = g + ((int64_t)b * T_len * H + h) * DK + dk0;
+    const T *kp = k + ((int64_t)b * T_len * H + h) * DK + dk0;
+    const T *qp = q + ((int64_t)b * T_len * H + h) * DK + dk0;
+    const T *vp = v + ((int64_t)b * T_len * H + h) * DV + dv0;
+    TO *op = out + ((int64_t)b * T_len * H + h) * DV + dv0;
+
+    struct Step {
+        RawVec<float, RK> g;
+        RawVec<T, RK> k, q;
+        RawVec<T, 4> v;
+    };
+    auto load_step = [&](Step &s, int step) {
+        int t = reverse ? T_len - 1 - step : step;
+        s.g.load(gp + t * strideK);
+        s.k.load(kp + t * strideK);
+        s.q.load(qp + t * strideK);
+        s.v.load(vp + t * strideV);
+    };
+    auto compute = [&](const Step &s, int step) {
+        int t = reverse ? T_len - 1 - step : step;
+        float vv[4], o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) vv[j] = s.v.get(j);
+#pragma unroll
+        for (int i = 0; i < RK; ++i) {
+            float f = __expf(s.g.get(i)), ki = s.k.get(i), qi = s.q.get(i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                S[i][j] = f * S[i][j] + ki * vv[j];
+                o[j] += qi * S[i][j];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = reduce_over_c(o[j]);
+        if (c == 0) store_vec<TO, 4>(op + t * strideV, o);
+    };
+
+    Step cur[U], nxt[U];
+    const int nblk = T_len / U;
+    if (nblk > 0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) load_step(cur[u], u);
+    }
+    for (int blk = 0; blk < nblk; ++blk) {
+        if (blk + 1 < nblk) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) load_step(nxt[u], (blk + 1) * U + u);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) compute(cur[u], blk * U + u);
+#pragma unroll
+        for (int u = 0; u < U; ++u) cur[u] = nxt[u];
+    }
+    for (int step = nblk * U; step < T_len; ++step) {
+        load_step(cur[0], step);
+        compute(cur[0], step);
+    }
+    {
+        T *hp = hT + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+#pragma unroll
+        for (int i = 0; i < RK; ++i) store_vec<T, 4>(hp + (int64_t)i * DV, S[i]);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward, sweep 1 (same time direction as the forward): recompute S_t, dq_t = S_t do_t.
+// Block = DK/16 waves = one (b,h); wave w owns state rows [16w, 16w+16); lane (a, c) owns rows
+// 16w + [4a, 4a+4) x columns [c*RV, (c+1)*RV).  Writes dq and, into the d(log_fgate) buffer, q*dq
+// in fp32 for sweep 2.
+// ------------------------------------------------------------------------------------------------
+template <typename T, typename TO, int RV, int U>
+__global__ __launch_bounds__(RV * 64) void recurrent_bwd_dq_kernel(
+    const T *__restrict__ h0, const float *__restrict__ g, const T *__restrict__ v,
+    const T *__restrict__ k, const T *__restrict__ q, const TO *__restrict__ dout,
+    T *__restrict__ dq, float *__restrict__ qdq, int T_len, int H, int reverse)
+{
+    constexpr int DV = RV * 16, DK = DV;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int a = lane & 3, c = lane >> 2;
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int dk0 = wave * 16 + a * 4, dv0 = c * RV;
+    const int64_t bh = (int64_t)b * H + h;
+
+    float S[4][RV];
+    {
+        const T *hp = h0 + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_vec<T, RV>(hp + (int64_t)i * DV, S[i]);
+    }
+    const int64_t strideK = (int64_t)H * DK, strideV = (int64_t)H * DV;
+    const int64_t offK = ((int64_t)b * T_len * H + h) * DK + dk0;
+    const int64_t offV = ((int64_t)b * T_len * H + h) * DV + dv0;
+
+    struct Step {
+        RawVec<float, 4> g;
+        RawVec<T, 4> k, q;
+        RawVec<T, RV> v;
+        RawVec<TO, RV> d;
+    };
+    auto load_step = [&](Step &s, int step) {
+        int t = reverse ? T_len - 1 - step : step;
+        s.g.load(g + offK + t * strideK);
+        s.k.load(k + offK + t * strideK);
+        s.q.load(q + offK + t * strideK);
+        s.v.load(v + offV + t * strideV);
+        s.d.load(dout + offV + t * strideV);
+    };
+    auto compute = [&](const Step &s, int step) {
+        int t = reverse ? T_len - 1 - step : step;
+        float acc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float f = __expf(s.g.get(i)), ki = s.k.get(i);
+            acc[i] = 0.f;
+#pragma unroll
+            for (int j = 0; j < RV; ++j) {
+                S[i][j] = f * S[i][j] + ki * s.v.get(j);
+                acc[i] += S[i][j] * s.d.get(j);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = reduce_over_c(acc[i]);
+        if (c == 0) {
+            float w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w[i] = acc[i] * s.q.get(i);
+            store_vec<T, 4>(dq + offK + t * strideK, acc);
+            store_vec<float, 4>(qdq + offK + t * strideK, w);
+        }
+    };
+
+    Step cur[U], nxt[U];
+    const int nblk = T_len / U;
+    if (nblk > 0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) load_step(cur[u], u);
+    }
+    for (int blk = 0; blk < nblk; ++blk) {
+        if (blk + 1 < nblk) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) load_step(nxt[u], (blk + 1) * U + u);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) compute(cur[u], blk * U + u);
+#pragma unroll
+        for (int u = 0; u < U; ++u) cur[u] = nxt[u];
+    }
+    for (int step = nblk * U; step < T_len; ++step) {
+        load_step(cur[0], step);
+        compute(cur[0], step);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward, sweep 2 (against the forward's time direction), same tiling as sweep 1:
+//   dS = dcarry + q_t do_t^T ; dk_t = dS v_t ; dv_t = dS^T k_t ; dcarry = exp(g_t) * dS
+//   dg_t = sum_{s>=t}(q_s*dq_s - k_s*dk_s) + sum_v(dhT * hT)                      (gla.py:263)
+// dv_t needs a sum over all DK rows, i.e. over the waves of the block: the per-wave partial sums of
+// TB steps are parked in LDS and combined once per TB steps.
+// ------------------------------------------------------------------------------------------------
+template <typename T, typename TO, int RV, int TB>
+__global__ __launch_bounds__(RV * 64) void recurrent_bwd_rev_kernel(
+    const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k,
+    const T *__restrict__ q, const T *__restrict__ hT, const T *__restrict__ dhT,
+    const TO *__restrict__ dout, T *__restrict__ dh0, float *__restrict__ dg, T *__restrict__ dv,
+    T *__restrict__ dk, int T_len, int H, int reverse)
+{
+    constexpr int DV = RV * 16, DK = DV, NW = RV;
+    __shared__ float part[TB * NW * DV];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int a = lane & 3, c = lane >> 2;
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int dk0 = wave * 16 + a * 4, dv0 = c * RV;
+    const int64_t bh = (int64_t)b * H + h;
+
+    float D[4][RV], fin[4], run[4];
+    {
+        const T *dp = dhT + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+        const T *hp = hT + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float hv[RV];
+            load_vec<T, RV>(dp + (int64_t)i * DV, D[i]);
+            load_vec<T, RV>(hp + (int64_t)i * DV, hv);
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < RV; ++j) s += D[i][j] * hv[j];
+            fin[i] = reduce_over_c(s);
+            run[i] = 0.f;
+        }
+    }
+    const int64_t strideK = (int64_t)H * DK, strideV = (int64_t)H * DV;
+    const int64_t offK = ((int64_t)b * T_len * H + h) * DK + dk0;
+    const int64_t offV = ((int64_t)b * T_len * H + h) * DV + dv0;
+    const int64_t offVrow = ((int64_t)b * T_len * H + h) * DV;
+
+    struct Step {
+        RawVec<float, 4> g, w;
+        RawVec<T, 4> k, q;
+        RawVec<T, RV> v;
+        RawVec<TO, RV> d;
+    };
+    // logical step s counts along the forward's direction; this sweep walks s = T-1 .. 0
+    auto phys = [&](int s) { return reverse ? T_len - 1 - s : s; };
+    auto load_step = [&](Step &s, int step) {
+        int t = phys(step);
+        s.g.load(g + offK + t * strideK);
+        s.w.load(dg + offK + t * strideK);
+        s.k.load(k + offK + t * strideK);
+        s.q.load(q + offK + t * strideK);
+        s.v.load(v + offV + t * strideV);
+        s.d.load(dout + offV + t * strideV);
+    };
+    auto compute = [&](const Step &s, int step, int slot) {
+        int t = phys(step);
+        float dkk[4], dvv[RV];
+#pragma unroll
+        for (int j = 0; j < RV; ++j) dvv[j] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float f = __expf(s.g.get(i)), ki = s.k.get(i), qi = s.q.get(i);
+            dkk[i] = 0.f;
+#pragma unroll
+            for (int j = 0; j < RV; ++j) {
+                float d = D[i][j] + qi * s.d.get(j);
+                dkk[i] += d * s.v.get(j);
+                dvv[j] += ki * d;
+                D[i][j] = f * d;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dkk[i] = reduce_over_c(dkk[i]);
+#pragma unroll
+        for (int j = 0; j < RV; ++j) dvv[j] = reduce_over_a(dvv[j]);
+        if (a == 0) {
+            float *pp = part + ((size_t)slot * NW + wave) * DV + dv0;
+#pragma unroll
+            for (int j = 0; j < RV; ++j) pp[j] = dvv[j];
+        }
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            run[i] += s.w.get(i) - dkk[i] * s.k.get(i);
+            o[i] = run[i] + fin[i];
+        }
+        if (c == 0) {
+            store_vec<T, 4>(dk + offK + t * strideK, dkk);
+            store_vec<float, 4>(dg + offK + t * strideK, o);
+        }
+    };
+    auto flush = [&](int first_step, int count) {
+        // steps first_step, first_step-1, ... live in slots 0..count-1
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < count * DV; idx += blockDim.x) {
+            int slot = idx / DV, col = idx % DV;
+            float s = 0.f;
+            for (int w = 0; w < NW; ++w) s += part[((size_t)slot * NW + w) * DV + col];
+            int t = phys(first_step - slot);
+            Elem<T>::store(dv + offVrow + t * strideV + col, s);
+        }
+        __syncthreads();
+    };
+
+    Step cur[TB], nxt[TB];
+    const int nblk = T_len / TB;
+    const int tail = T_len - nblk * TB;
+    // the tail (highest logical steps not filling a block) goes first, one step at a time
+    for (int i = 0; i < tail; ++i) {
+        int step = T_len - 1 - i;
+        load_step(cur[0], step);
+        compute(cur[0], step, 0);
+        flush(step, 1);
+    }
+    const int top = nblk * TB - 1;
+    if (nblk > 0) {
+#pragma unroll
+        for (int u = 0; u < TB; ++u) load_step(cur[u], top - u);
+    }
+    for (int blk = 0; blk < nblk; ++blk) {
+        const int first = top - blk * TB;
+        if (blk + 1 < nblk) {
+#pragma unroll
+            for (int u = 0; u < TB; ++u) load_step(nxt[u], first - TB - u);
+        }
+#pragma unroll
+        for (int u = 0; u < TB; ++u) compute(cur[u], first - u, u);
+        flush(first, TB);
+#pragma unroll
+        for (int u = 0; u < TB; ++u) cur[u] = nxt[u];
+    }
+    {
+        T *dp = dh0 + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) store_vec<T, RV>(dp + (int64_t)i * DV, D[i]);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+template <typename T, typename TO>
+static int launch_fwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, int reverse,
+                      const void *h0, const float *g, const void *v, const void *k, const void *q,
+                      void *hT, void *out)
+{
+    dim3 grid(H, B), block(DV / 16 * 64);
+#define GLA_FWD_CASE(RK_, U_)                                                                        \
+    hipLaunchKernelGGL((recurrent_fwd_kernel<T, TO, RK_, U_>), grid, block, 0, st, (const T *)h0, g, \
+                       (const T *)v, (const T *)k, (const T *)q, (T *)hT, (TO *)out, T_len, H,       \
+                       reverse)
+    switch (DK / 16) {
+    case 1: GLA_FWD_CASE(1, 4); break;
+    case 2: GLA_FWD_CASE(2, 4); break;
+    case 4: GLA_FWD_CASE(4, 4); break;
+    case 8: GLA_FWD_CASE(8, 2); break;
+    default: return GLA_ERR_SHAPE;
+    }
+#undef GLA_FWD_CASE
+    return launch_status();
+}
+
+template <typename T, typename TO>
+static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, int reverse,
+                      const void *h0, const float *g, const void *v, const void *k, const void *q,
+                      const void *hT, const void *dhT, const void *dout, void *dh0, float *dg, void *dv,
+                      void *dk, void *dq)
+{
+    dim3 grid(H, B), block(DK / 16 * 64);
+#define GLA_BWD_CASE(RV_, U_, TB_)                                                                      \
+    do {                                                                                                \
+        hipLaunchKernelGGL((recurrent_bwd_dq_kernel<T, TO, RV_, U_>), grid, block, 0, st,               \
+                           (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,                  \
+                           (const TO *)dout, (T *)dq, dg, T_len, H, reverse);                           \
+        hipLaunchKernelGGL((recurrent_bwd_rev_kernel<T, TO, RV_, TB_>), grid, block, 0, st, g,          \
+                           (const T *)v, (const T *)k, (const T *)q, (const T *)hT, (const T *)dhT,     \
+                           (const TO *)dout, (T *)dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse);        \
+    } while (0)
+    switch (DV / 16) {
+    case 1: GLA_BWD_CASE(1, 4, 4); break;
+    case 2: GLA_BWD_CASE(2, 4, 4); break;
+    case 4: GLA_BWD_CASE(4, 4, 4); break;
+    case 8: GLA_BWD_CASE(8, 2, 2); break;
+    default: return GLA_ERR_SHAPE;
+    }
+#undef GLA_BWD_CASE
+    return launch_status();
+}
+
+static int check_recurrent(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, int dtype,
+                           int out_dtype)
+{
+    if (B <= 0 || T <= 0 || H <= 0 || DK <= 0 || DV <= 0) return GLA_ERR_SHAPE;
+    if (B > 65535 || H > 65535 || T > (1 << 30)) return GLA_ERR_SHAPE;
+    // the reference requires DK == DV for this path (gla.py:120, 391)
+    if (DK != DV || !(DK == 16 || DK == 32 || DK == 64 || DK == 128)) return GLA_ERR_SHAPE;
+    if (dtype != GLA_F32 && dtype != GLA_BF16) return GLA_ERR_DTYPE;
+    if (out_dtype != GLA_F32 && out_dtype != GLA_BF16) return GLA_ERR_DTYPE;
+    if (out_dtype == GLA_BF16 && dtype == GLA_F32) return GLA_ERR_DTYPE;
+    return GLA_OK;
+}
+
+}  // namespace gla
+
+extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                 gla_dtype dtype, gla_dtype out_dtype, int reverse,
+                                 const void *hidden_init, const float *log_fgate, const void *value,
+                                 const void *key, const void *query, void *hidden_final, void *out)
+{
+    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, out_dtype);
+    if (rc) return rc;
+    if (!hidden_init || !log_fgate || !value || !key || !query || !hidden_final || !out)
+        return GLA_ERR_NULL;
+    const void *ptrs[] = {hidden_init, log_fgate, value, key, query, hidden_final, out};
+    for (const void *p : ptrs)
+        if (!gla::aligned16(p)) return GLA_ERR_ALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == GLA_BF16 && out_dtype == GLA_BF16)
+        return gla::launch_fwd<__bf16, __bf16>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value,
+                                               key, query, hidden_final, out);
+    if (dtype == GLA_BF16)
+        return gla::launch_fwd<__bf16, float>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value,
+                                              key, query, hidden_final, out);
+    return gla::launch_fwd<float, float>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value, key,
+                                         query, hidden_final, out);
+}
+
+extern "C" int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                 gla_dtype dtype, gla_dtype out_dtype, int reverse,
+                                 const void *hidden_init, const float *log_fgate, const void *value,
+                                 const void *key, const void *query, const void *hidden_final,
+                                 const void *dhidden_final, const void *dout, void *dhidden_init,
+                                 float *dlog_fgate, void *dvalue, void *dkey, void *dquery)
+{
+    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, out_dtype);
+    if (rc) return rc;
+    const void *ptrs[] = {hidden_init, log_fgate, value, key, query, hidden_final, dhidden_final,
+                          dout, dhidden_init, dlog_fgate, dvalue, dkey, dquery};
+    for (const void *p : ptrs) {
+        if (!p) return GLA_ERR_NULL;
+        if (!gla::aligned16(p)) return GLA_ERR_ALIGN;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == GLA_BF16 && out_dtype == GLA_BF16)
+        return gla::launch_bwd<__bf16, __bf16>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value,
+                                               key, query, hidden_final, dhidden_final, dout, dhidden_init,
+                                               dlog_fgate, dvalue, dkey, dquery);
+    if (dtype == GLA_BF16)
+        return gla::launch_bwd<__bf16, float>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value,
+                                              key, query, hidden_final, dhidden_final, dout, dhidden_init,
+                                              dlog_fgate, dvalue, dkey, dquery);
+    return gla::launch_bwd<float, float>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value, key,
+                                         query, hidden_final, dhidden_final, dout, dhidden_init, dlog_fgate,
+                                         dvalue, dkey, dquery);
+}

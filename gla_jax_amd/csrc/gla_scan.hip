@@ -1,0 +1,160 @@
+// Stand-alone scans of the reference's ops.py as gfx950 kernels:
+//   gla_cumsum_f32    <- cumsum_recursive / cumsum_pallas / cumsum_kernel   (ops.py:152-284)
+//   gla_rnn_scan_f32  <- rnn_recursive / rnn_pallas / rnn_kernel            (ops.py:286-456)
+// Both are HBM-bound streaming kernels: lanes map to the contiguous inner axis so every wave access
+// is a full 256-byte row segment, and the scanned axis is walked by the wave in registers.
+#include "gla_common.hpp"
+
+namespace gla {
+
+// One block = one outer index x 64 consecutive inner columns.  The scanned axis is cut into WAVES
+// contiguous segments, one per wave: pass 1 sums each segment, the segment totals are prefixed
+// through LDS, pass 2 re-reads the segment (L2 hit) and writes the running sum.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void cumsum_kernel(const float *__restrict__ src,
+                                                            const float *__restrict__ init,
+                                                            float *__restrict__ dst, int64_t t_len,
+                                                            int64_t n_inner, int reverse)
+{
+    __shared__ float totals[WAVES][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t col = (int64_t)blockIdx.x * 64 + lane;
+    const int64_t outer = blockIdx.y;
+    const bool valid = col < n_inner;
+    const int64_t seg = (t_len + WAVES - 1) / WAVES;
+    const int64_t s0 = wave * seg;
+    const int64_t s1 = s0 + seg < t_len ? s0 + seg : t_len;
+    const float *base = src + outer * t_len * n_inner + col;
+    float *obase = dst + outer * t_len * n_inner + col;
+
+    float sum = 0.f;
+    if (valid) {
+        int64_t s = s0;
+        for (; s + 4 <= s1; s += 4) {
+            float a[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int64_t t = reverse ? t_len - 1 - (s + u) : s + u;
+                a[u] = base[t * n_inner];
+            }
+            sum += (a[0] + a[1]) + (a[2] + a[3]);
+        }
+        for (; s < s1; ++s) {
+            int64_t t = reverse ? t_len - 1 - s : s;
+            sum += base[t * n_inner];
+        }
+    }
+    totals[wave][lane] = sum;
+    __syncthreads();
+    if (!valid) return;
+    float run = init ? init[outer * n_inner + col] : 0.f;
+    for (int w = 0; w < wave; ++w) run += totals[w][lane];
+    int64_t s = s0;
+    for (; s + 4 <= s1; s += 4) {
+        float a[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            int64_t t = reverse ? t_len - 1 - (s + u) : s + u;
+            a[u] = base[t * n_inner];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            int64_t t = reverse ? t_len - 1 - (s + u) : s + u;
+            run += a[u];
+            obase[t * n_inner] = run;
+        }
+    }
+    for (; s < s1; ++s) {
+        int64_t t = reverse ? t_len - 1 - s : s;
+        run += base[t * n_inner];
+        obase[t * n_inner] = run;
+    }
+}
+
+// One thread = one (k, 4 consecutive v) strip of the state, walked over T in registers; the loads
+// of step n do not depend on the recurrence, so UNROLL of them are kept in flight.
+template <int UNROLL>
+__global__ __launch_bounds__(256) void rnn_scan_kernel(const float *__restrict__ a,
+                                                       const float *__restrict__ kv,
+                                                       const float *__restrict__ init_a,
+                                                       const float *__restrict__ init_kv,
+                                                       float *__restrict__ out_a,
+                                                       float *__restrict__ out_x, int64_t T, int64_t K,
+                                                       int64_t V, int reverse)
+{
+    const int64_t v4 = V / 4;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= K * v4) return;
+    const int64_t b = blockIdx.y;
+    const int64_t k = idx / v4, vq = idx % v4;
+    const float *ab = a + b * T * K + k;
+    const f32x4 *xb = reinterpret_cast<const f32x4 *>(kv + b * T * K * V + k * V) + vq;
+    f32x4 *ob = reinterpret_cast<f32x4 *>(out_x + b * T * K * V + k * V) + vq;
+    float *oab = out_a ? out_a + b * T * K + k : nullptr;
+    f32x4 x = {0.f, 0.f, 0.f, 0.f};
+    if (init_kv) x = reinterpret_cast<const f32x4 *>(init_kv + b * K * V + k * V)[vq];
+    float ca = init_a ? init_a[b * K + k] : 0.f;
+    int64_t s = 0;
+    for (; s + UNROLL <= T; s += UNROLL) {
+        float av[UNROLL];
+        f32x4 bv[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int64_t t = reverse ? T - 1 - (s + u) : s + u;
+            av[u] = ab[t * K];
+            bv[u] = xb[t * K * v4];
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int64_t t = reverse ? T - 1 - (s + u) : s + u;
+            float f = __expf(av[u]);
+            x = f * x + bv[u];
+            ca += av[u];
+            ob[t * K * v4] = x;
+            if (oab && vq == 0) oab[t * K] = ca;
+        }
+    }
+    for (; s < T; ++s) {
+        int64_t t = reverse ? T - 1 - s : s;
+        float av = ab[t * K];
+        x = __expf(av) * x + xb[t * K * v4];
+        ca += av;
+        ob[t * K * v4] = x;
+        if (oab && vq == 0) oab[t * K] = ca;
+    }
+}
+
+}  // namespace gla
+
+extern "C" int gla_cumsum_f32(void *stream, const float *src, const float *init, float *dst,
+                              int64_t n_outer, int64_t t_len, int64_t n_inner, int reverse)
+{
+    if (!src || !dst) return GLA_ERR_NULL;
+    if (n_outer <= 0 || t_len <= 0 || n_inner <= 0 || n_outer > 65535) return GLA_ERR_SHAPE;
+    dim3 grid((unsigned)((n_inner + 63) / 64), (unsigned)n_outer);
+    hipStream_t st = (hipStream_t)stream;
+    if (t_len >= 64)
+        hipLaunchKernelGGL(gla::cumsum_kernel<4>, grid, dim3(256), 0, st, src, init, dst, t_len, n_inner,
+                           reverse);
+    else
+        hipLaunchKernelGGL(gla::cumsum_kernel<1>, grid, dim3(64), 0, st, src, init, dst, t_len, n_inner,
+                           reverse);
+    return gla::launch_status();
+}
+
+extern "C" int gla_rnn_scan_f32(void *stream, const float *log_fgate, const float *kv,
+                                const float *init_log_fgate, const float *init_kv,
+                                float *out_log_lambda, float *out_state, int64_t batch, int64_t T,
+                                int64_t K, int64_t V, int reverse)
+{
+    if (!log_fgate || !kv || !out_state) return GLA_ERR_NULL;
+    if (batch <= 0 || T <= 0 || K <= 0 || V <= 0 || V % 4 != 0 || batch > 65535) return GLA_ERR_SHAPE;
+    if (!gla::aligned16(kv) || !gla::aligned16(out_state) || (init_kv && !gla::aligned16(init_kv)))
+        return GLA_ERR_ALIGN;
+    int64_t n = K * (V / 4);
+    dim3 grid((unsigned)((n + 255) / 256), (unsigned)batch);
+    hipLaunchKernelGGL(gla::rnn_scan_kernel<8>, grid, dim3(256), 0, (hipStream_t)stream, log_fgate, kv,
+                       init_log_fgate, init_kv, out_log_lambda, out_state, T, K, V, reverse);
+    return gla::launch_status();
+}

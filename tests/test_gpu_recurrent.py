@@ -1,0 +1,94 @@
+"""GPU parity of recurrent_gla / recurrent_gla_naive (forward, all five gradients) through the C ABI
+against the oracle.  Tolerance (north_star): max|err| / RMS(oracle) <= 2e-2 for bf16 inputs,
+<= 1e-4 for fp32."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gla_oracle as O
+from oracle import naive_c
+from tests.util import TOL, assert_close, cotangents, gpu_inputs, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def run_fwd_bwd(fn, dev, dhT, dout, out_dtype, **kw):
+    dev = [t.clone().requires_grad_(True) for t in dev]
+    hT, out = fn(*dev, **kw)
+    loss = (hT.float() * dhT.float()).sum() + (out.float() * dout.float()).sum()
+    grads = torch.autograd.grad(loss, dev)
+    return hT, out, grads
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B,T,H,D", [(2, 67, 3, 64), (1, 32, 2, 16), (1, 40, 1, 128), (2, 24, 2, 32)])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_recurrent_gla_matches_oracle(dtype, B, T, H, D, reverse):
+    from gla_jax_amd import recurrent_gla
+    (h0, g, v, k, q), dev = gpu_inputs(B, T, H, D, 3.0, seed=B * 100 + T, dtype=dtype)
+    dhT, dout = cotangents(h0, v, 1, dtype)
+    hT, out, grads = run_fwd_bwd(recurrent_gla, dev, to_dev(dhT, dtype), to_dev(dout, dtype), dtype,
+                                 reverse=reverse)
+    assert out.dtype == dtype and hT.dtype == dtype
+    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=reverse)
+    tol = TOL[dtype]
+    assert_close("out", to_np(out), exp[6], tol, stored=dtype)
+    assert_close("hidden_final", to_np(hT), exp[5], tol, stored=dtype)
+    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
+                                (dtype, torch.float32, dtype, dtype, dtype)):
+        assert_close(name, to_np(got), e, tol, stored=st)
+
+
+def test_recurrent_gla_naive_returns_fp32_out():
+    from gla_jax_amd import recurrent_gla_naive
+    dtype = torch.bfloat16
+    (h0, g, v, k, q), dev = gpu_inputs(2, 50, 2, 64, 5.0, seed=9, dtype=dtype)
+    dhT, dout = cotangents(h0, v, 2, torch.float32)
+    dhT = O.bf16_round(dhT)
+    hT, out, grads = run_fwd_bwd(recurrent_gla_naive, dev, to_dev(dhT, dtype), to_dev(dout, torch.float32),
+                                 torch.float32, reverse=False)
+    assert out.dtype == torch.float32 and hT.dtype == dtype            # gla.py:37, 46
+    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout)
+    assert_close("out", to_np(out), exp[6], 1e-4)                      # fp32 state and output
+    assert_close("hidden_final", to_np(hT), exp[5], TOL[dtype], stored=dtype)
+    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
+                                (dtype, torch.float32, dtype, dtype, dtype)):
+        assert_close(name, to_np(got), e, TOL[dtype], stored=st)
+
+
+def test_recurrent_unbatched_and_vmap_agree():
+    from gla_jax_amd import recurrent_gla
+    (h0, g, v, k, q), dev = gpu_inputs(3, 33, 2, 64, 3.0, seed=4, dtype=torch.bfloat16)
+    hT_b, out_b = recurrent_gla(*dev)
+    hT_v, out_v = torch.func.vmap(recurrent_gla)(*dev)
+    assert torch.equal(hT_b, hT_v) and torch.equal(out_b, out_v)
+    for b in range(3):
+        hT_1, out_1 = recurrent_gla(*[t[b] for t in dev])
+        assert torch.equal(hT_1, hT_b[b]) and torch.equal(out_1, out_b[b])
+
+
+def test_recurrent_full_benchmark_shape_against_c_oracle():
+    """BASELINE configs[4]: B16,T2048,H16,D64 bf16, gates log_sigmoid(3+N(0,1)); forward and all
+    gradients against the C restatement in fp64 on every (b,h) pair."""
+    from gla_jax_amd import recurrent_gla
+    dtype = torch.bfloat16
+    B, T, H, D = 16, 2048, 16, 64
+    (h0, g, v, k, q), dev = gpu_inputs(B, T, H, D, 3.0, seed=44, dtype=dtype)
+    dhT, dout = cotangents(h0, v, 3, dtype)
+    hT, out, grads = run_fwd_bwd(recurrent_gla, dev, to_dev(dhT, dtype), to_dev(dout, dtype), dtype)
+    exp = naive_c.naive_bwd(h0, g, v, k, q, dhT, dout, dtype=np.float64, nthreads=16)
+    tol = TOL[dtype]
+    assert_close("out", to_np(out), exp[6], tol, stored=dtype)
+    assert_close("hidden_final", to_np(hT), exp[5], tol, stored=dtype)
+    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
+                                (dtype, torch.float32, dtype, dtype, dtype)):
+        assert_close(name, to_np(got), e, tol, stored=st)
+
+
+def test_recurrent_rejects_bad_arguments():
+    from gla_jax_amd import _lib, recurrent_gla
+    (h0, g, v, k, q), dev = gpu_inputs(1, 8, 1, 48, 3.0, seed=5, dtype=torch.bfloat16)
+    with pytest.raises(_lib.GlaError):
+        recurrent_gla(*dev)                       # head dim 48 is not built
+    with pytest.raises(AssertionError):
+        recurrent_gla(dev[0], dev[1], dev[2][..., :32], dev[3], dev[4])
