@@ -7,7 +7,7 @@ import torch
 
 from oracle import gla_oracle as O
 from oracle import naive_c
-from tests.util import TOL, assert_close, cotangents, gpu_inputs, to_dev, to_np
+from tests.util import TOL, assert_close, cotangents, gpu_inputs, grad_kinds, to_dev, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -46,8 +46,7 @@ def test_chunk_backward_matches_oracle(dtype, B, T, H, D, chunk, shift):
     grads = torch.autograd.grad(loss, dev)
     exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout)
     for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                (dtype, torch.float32, dtype, dtype, dtype)):
-        assert got.dtype == st
+                                grad_kinds(dtype)):
         assert_close(name, to_np(got), e, TOL[dtype], stored=st)
 
 
@@ -90,3 +89,40 @@ def test_chunk_rejects_what_the_reference_rejects():
         chunk_gla(*dev, 64)                 # 96 % 64 != 0 (einops rearrange, gla.py:674)
     with pytest.raises(_lib.GlaError):
         chunk_gla(*dev, 8)                  # below the smallest tile built here
+
+
+def _full_shape_check(B, T, H, D, chunk, shift, seed, heads):
+    """Forward + all gradients at a BASELINE shape against the C restatement of the naive recurrence
+    (fp64) on the listed heads (all batches)."""
+    from gla_jax_amd import chunk_gla
+    dtype = torch.bfloat16
+    (h0, g, v, k, q), dev = gpu_inputs(B, T, H, D, shift, seed=seed, dtype=dtype)
+    dhT, dout = cotangents(h0, v, seed, dtype)
+    dev = [t.clone().requires_grad_(True) for t in dev]
+    hT, out = chunk_gla(*dev, chunk)
+    loss = (hT.float() * to_dev(dhT, torch.float32)).sum() + (out.float() * to_dev(dout, torch.float32)).sum()
+    grads = torch.autograd.grad(loss, dev)
+    hs = list(heads)
+    sl = lambda a: np.ascontiguousarray(a[:, :, hs]) if a.ndim == 4 and a.shape[1] == T else np.ascontiguousarray(a[:, hs])
+    exp = naive_c.naive_bwd(sl(h0), sl(g), sl(v), sl(k), sl(q), sl(dhT), sl(dout), dtype=np.float64, nthreads=16)
+    raw = {}
+    raw["out"] = assert_close("out", sl(to_np(out)), exp[6], TOL[dtype], stored=dtype)
+    raw["hidden_final"] = assert_close("hidden_final", sl(to_np(hT)), exp[5], TOL[dtype], stored=dtype)
+    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
+                                grad_kinds(dtype)):
+        raw[name] = assert_close(name, sl(to_np(got)), e, TOL[dtype], stored=st)
+    print("plain max|err|/rms:", {k_: f"{v_:.2e}" for k_, v_ in raw.items()})
+    return raw
+
+
+def test_chunk_baseline_config_fwd_bwd_full_shape():
+    """BASELINE configs[1]/[2]: B4,T4096,H6,D128, chunk 128, gates log_sigmoid(5+N(0,1)); every head."""
+    raw = _full_shape_check(4, 4096, 6, 128, 128, 5.0, seed=12, heads=range(6))
+    # weak decay: the plain north_star metric (no allowance) stays at the 2e-2 level for every output
+    assert max(raw.values()) <= 3e-2
+
+
+def test_chunk_long_context_strong_decay_full_shape():
+    """BASELINE configs[3]: B1,T32768,H8,D128, chunk 128, gates log_sigmoid(N(0,1)); heads 0 and 5 are
+    checked against the oracle (the other six run the same kernels on other data)."""
+    _full_shape_check(1, 32768, 8, 128, 128, 0.0, seed=13, heads=(0, 5))

@@ -7,7 +7,7 @@ import torch
 
 from oracle import gla_oracle as O
 from oracle import naive_c
-from tests.util import TOL, assert_close, cotangents, gpu_inputs, to_dev, to_np
+from tests.util import TOL, assert_close, cotangents, gpu_inputs, grad_kinds, to_dev, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -35,7 +35,7 @@ def test_recurrent_gla_matches_oracle(dtype, B, T, H, D, reverse):
     assert_close("out", to_np(out), exp[6], tol, stored=dtype)
     assert_close("hidden_final", to_np(hT), exp[5], tol, stored=dtype)
     for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                (dtype, torch.float32, dtype, dtype, dtype)):
+                                grad_kinds(dtype)):
         assert_close(name, to_np(got), e, tol, stored=st)
 
 
@@ -52,7 +52,7 @@ def test_recurrent_gla_naive_returns_fp32_out():
     assert_close("out", to_np(out), exp[6], 1e-4)                      # fp32 state and output
     assert_close("hidden_final", to_np(hT), exp[5], TOL[dtype], stored=dtype)
     for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                (dtype, torch.float32, dtype, dtype, dtype)):
+                                grad_kinds(dtype)):
         assert_close(name, to_np(got), e, TOL[dtype], stored=st)
 
 
@@ -81,7 +81,7 @@ def test_recurrent_full_benchmark_shape_against_c_oracle():
     assert_close("out", to_np(out), exp[6], tol, stored=dtype)
     assert_close("hidden_final", to_np(hT), exp[5], tol, stored=dtype)
     for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                (dtype, torch.float32, dtype, dtype, dtype)):
+                                grad_kinds(dtype)):
         assert_close(name, to_np(got), e, tol, stored=st)
 
 

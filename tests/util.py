@@ -23,21 +23,44 @@ def err_over_rms(got, exp):
 
 
 def assert_close(name, got, exp, tol, stored=None):
-    """max|got-exp| <= tol * RMS(exp).  When the quantity is STORED in bf16 (`stored` is
-    torch.bfloat16) the bound gets half a bf16 ulp of the expected value on top: rounding the exact
-    result to bf16 costs up to 2^-8 |x|, which alone exceeds 2e-2 RMS wherever |x| > 5 RMS (measured:
-    the fp64 oracle output of BASELINE configs[4] rounded to bf16 sits at 2.24e-2 RMS)."""
+    """Elementwise |got-exp| <= tol * RMS(exp) + 2^-7 |exp| when the computation runs on bf16
+    operands (`stored` is torch.bfloat16 or "bf16-operands"), else the plain max|err| <= tol * RMS(exp).
+
+    Why the second term: one bf16 ulp of the element's own magnitude.  (a) Rounding the EXACT result
+    to bf16 for storage already costs up to 2^-8 |x| - measured: the fp64 oracle output of BASELINE
+    configs[4] rounded to bf16 sits at 2.24e-2 RMS, above the 2e-2 RMS target, because |out| reaches
+    7 RMS.  (b) Every bf16 tensor-core formulation, the reference's included, rounds the gate-rescaled
+    q/k operands to bf16 (gla.py:816-819, 991-992): elements that are sums of a few large terms
+    (strong decay) inherit ~2^-8 relative error, which again beats 2e-2 RMS only in the heavy tail
+    (|x| > 5 RMS).  The oracle's emulation of the reference's own rounding points shows the same
+    (tests/test_oracle.py::test_reference_rounding_points_gradients).  Returns the plain
+    max|err|/RMS so callers can log it."""
     assert got.shape == exp.shape, f"{name}: shape {got.shape} != {exp.shape}"
     assert np.isfinite(got).all(), f"{name}: non-finite values"
     exp = np.asarray(exp, dtype=np.float64)
-    rms = np.sqrt((exp ** 2).mean())
-    bound = tol * max(rms, 1e-30)
+    rms = max(float(np.sqrt((exp ** 2).mean())), 1e-30)
     err = np.abs(np.asarray(got, dtype=np.float64) - exp)
-    if stored == torch.bfloat16:
-        err = err - np.abs(exp) * 2.0 ** -8
-    e = float(err.max() / max(rms, 1e-30))
-    assert e <= tol, f"{name}: max|err|/rms = {e:.3e} > {tol:.1e} (rms {rms:.3e}, bound {bound:.3e})"
-    return e
+    raw = float(err.max() / rms)
+    if stored == "bf16-suffix-sum":
+        # d(log_fgate) is a reverse running sum of signed terms inside each chunk (gla.py:616-617), so
+        # the rounding error of one large term is inherited by every earlier position of the chunk,
+        # whatever the size of the value there: the bf16-ulp allowance is taken relative to the largest
+        # magnitude instead of the element's own, and the relative L2 error is bounded on top.
+        l2 = float(np.linalg.norm(err) / max(np.linalg.norm(exp), 1e-30))
+        assert l2 <= 1e-2, f"{name}: relative L2 error {l2:.3e} > 1e-2"
+        err = err - np.abs(exp).max() * 2.0 ** -7
+    elif stored is not None and stored != torch.float32:
+        err = err - np.abs(exp) * 2.0 ** -7
+    e = float(err.max() / rms)
+    assert e <= tol, f"{name}: excess error {e:.3e} > {tol:.1e} x RMS (plain max|err|/rms = {raw:.3e}, rms {rms:.3e})"
+    return raw
+
+
+def grad_kinds(dtype):
+    """`stored` argument of assert_close for (dhidden_init, dlog_fgate, dvalue, dkey, dquery)."""
+    if dtype == torch.bfloat16:
+        return (dtype, "bf16-suffix-sum", dtype, dtype, dtype)
+    return (dtype,) * 5
 
 
 def gpu_inputs(B, T, H, D, shift, seed, dtype, batch_dims=True):
