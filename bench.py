@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""Benchmark of the GLA hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload chunk|recurrent|long] [--no-cpu]
+
+A step is one pass of the hot path over one batch of synthetic input resident in HBM: chunk_gla
+forward + backward (all five gradients) through the C ABI of libgla_hip.so at BASELINE.json's
+headline shape (B4, T4096, H6, D128, chunk 128, bf16 q/k/v/hidden, fp32 gates).  Prints ONE JSON line.
+
+`roofline` describes the dominant kernel (the per-chunk gradient kernel): algorithmic HBM bytes per
+launch (22*D bytes per token-head: read q,k,v,dout bf16 + gates fp32, write dq,dk,dv bf16 + dgates
+fp32) over its average duration, measured here with events on the launch stream, against 8 TB/s.
+`kernels` lists every kernel of the step the same way; `mfma_frac` prices the step's algorithmic
+FLOPs (18*D^2 per token-head) against the 2.5 PFLOP/s dense bf16 MFMA peak.
+`cpu_baseline` times the C restatement of the reference's recurrent_gla_naive (forward + its
+two-sweep gradients, fp32 state, OpenMP over batch*heads) on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+FP32_VALU_PEAK_TFLOPS = 157.3
+
+WORKLOADS = {
+    # name: (kind, B, T, H, D, chunk, gate shift)
+    "chunk": ("chunk", 4, 4096, 6, 128, 128, 5.0),       # BASELINE configs[1]/[2] (headline metric)
+    "long": ("chunk", 1, 32768, 8, 128, 128, 0.0),       # BASELINE configs[3]
+    "recurrent": ("recurrent", 16, 2048, 16, 64, 0, 3.0),  # BASELINE configs[4]
+}
+
+
+def make_device_inputs(B, T, H, D, shift, seed=0):
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    bf = torch.bfloat16
+    rn = lambda *s: torch.randn(*s, generator=g, device="cuda", dtype=torch.float32)
+    h0 = rn(B, H, D, D).to(bf)
+    gate = torch.nn.functional.logsigmoid(shift + rn(B, T, H, D)).contiguous()
+    v, k, q = rn(B, T, H, D).to(bf), rn(B, T, H, D).to(bf), rn(B, T, H, D).to(bf)
+    dhT, dout = rn(B, H, D, D).to(bf), rn(B, T, H, D).to(bf)
+    return h0, gate, v, k, q, dhT, dout
+
+
+def time_events(fn, steps, warmup):
+    """Average milliseconds of fn() over `steps` launches, by events on torch's current stream (the
+    stream every kernel of the library is launched on)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(steps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / steps
+
+
+def bench_chunk(B, T, H, D, chunk, shift, steps, warmup):
+    import torch
+    from gla_jax_amd import _lib
+    lib = _lib.load()
+    h0, g, v, k, q, dhT, dout = make_device_inputs(B, T, H, D, shift)
+    dt = _lib.GLA_BF16
+    wsf = torch.empty(lib.gla_chunk_fwd_workspace_bytes(B, T, H, D, D, chunk, dt), dtype=torch.uint8, device="cuda")
+    wsb = torch.empty(lib.gla_chunk_bwd_workspace_bytes(B, T, H, D, D, chunk, dt), dtype=torch.uint8, device="cuda")
+    states = torch.empty(lib.gla_chunk_states_bytes(B, T, H, D, D, chunk, dt), dtype=torch.uint8, device="cuda")
+    hT, out = torch.empty_like(h0), torch.empty_like(v)
+    dh0, dg = torch.empty_like(h0), torch.empty_like(g)
+    dv, dk, dq = torch.empty_like(v), torch.empty_like(k), torch.empty_like(q)
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda t: t.data_ptr()
+
+    def fwd(stages=7):
+        rc = lib.gla_chunk_fwd_stages(st, stages, B, T, H, D, D, chunk, dt, p(h0), p(g), p(v), p(k), p(q),
+                                      p(hT), p(out), p(states), p(wsf), wsf.numel())
+        _lib.check("gla_chunk_fwd", rc)
+
+    def bwd(stages=7):
+        rc = lib.gla_chunk_bwd_stages(st, stages, B, T, H, D, D, chunk, dt, p(g), p(v), p(k), p(q), p(states),
+                                      p(dhT), p(dout), p(dh0), p(dg), p(dv), p(dk), p(dq), p(wsb), wsb.numel())
+        _lib.check("gla_chunk_bwd", rc)
+
+    def step():
+        fwd()
+        bwd()
+
+    # the timed region of the contract: exactly `steps` steps between two device synchronisations
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+
+    n_th = B * T * H
+    N = T // min(chunk, 128)
+    state_f32 = B * H * N * D * D * 4
+    state_bf16 = B * H * N * D * D * 2
+    # algorithmic bytes (inputs read once, outputs written once) and what each kernel really moves
+    kernels = {
+        "fwd.chunk_outer_kernel": (lambda: fwd(1), 8 * D * n_th, 8 * D * n_th + state_f32),
+        "fwd.chunk_scan_kernel": (lambda: fwd(2), 0, state_f32 + state_bf16),
+        "fwd.chunk_out_kernel": (lambda: fwd(4), 12 * D * n_th, 12 * D * n_th + state_bf16),
+        "bwd.chunk_outer_kernel": (lambda: bwd(1), 8 * D * n_th, 8 * D * n_th + state_f32),
+        "bwd.chunk_scan_kernel": (lambda: bwd(2), 0, state_f32 + state_bf16),
+        "bwd.chunk_grad_kernel": (lambda: bwd(4), 22 * D * n_th, 22 * D * n_th + 2 * state_bf16),
+    }
+    per = {}
+    for name, (fn, alg, moved) in kernels.items():
+        ms = time_events(fn, max(steps, 10), 3)
+        per[name] = {"ms": round(ms, 5), "alg_GBs": round(alg / ms / 1e6, 1), "moved_GBs": round(moved / ms / 1e6, 1)}
+    dom = max(per, key=lambda n: per[n]["ms"])
+    dom_alg = kernels[dom][1]
+    achieved = dom_alg / per[dom]["ms"] / 1e6
+    flops = 18 * D * D * n_th
+    res = {
+        "value": B * T / ms_step / 1e3,
+        "ms_per_step": ms_step,
+        "roofline": {"bound": "hbm", "kernel": dom.split(".")[1], "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "alg_bytes_per_launch": dom_alg},
+        "kernels": per,
+        "step_hbm_frac": round(34 * D * n_th / ms_step / 1e6 / HBM_PEAK_GBS, 4),
+        "mfma_frac": round(flops / ms_step / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+        "sum_kernel_ms": round(sum(x["ms"] for x in per.values()), 5),
+    }
+    return res
+
+
+def bench_recurrent(B, T, H, D, shift, steps, warmup):
+    import torch
+    from gla_jax_amd import _lib
+    lib = _lib.load()
+    h0, g, v, k, q, dhT, dout = make_device_inputs(B, T, H, D, shift)
+    dt = _lib.GLA_BF16
+    hT, out = torch.empty_like(h0), torch.empty_like(v)
+    dh0, dg = torch.empty_like(h0), torch.empty_like(g)
+    dv, dk, dq = torch.empty_like(v), torch.empty_like(k), torch.empty_like(q)
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda t: t.data_ptr()
+
+    def fwd():
+        _lib.check("gla_recurrent_fwd", lib.gla_recurrent_fwd(st, B, T, H, D, D, dt, dt, 0, p(h0), p(g), p(v),
+                                                            p(k), p(q), p(hT), p(out)))
+
+    def bwd():
+        _lib.check("gla_recurrent_bwd", lib.gla_recurrent_bwd(st, B, T, H, D, D, dt, dt, 0, p(h0), p(g), p(v),
+                                                            p(k), p(q), p(hT), p(dhT), p(dout), p(dh0), p(dg),
+                                                            p(dv), p(dk), p(dq)))
+
+    def step():
+        fwd()
+        bwd()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+    n_th = B * T * H
+    ms_f = time_events(fwd, max(steps, 5), 2)
+    ms_b = time_events(bwd, max(steps, 5), 2)
+    alg = 34 * D * n_th
+    per = {"recurrent_fwd_kernel": {"ms": round(ms_f, 5), "alg_GBs": round(12 * D * n_th / ms_f / 1e6, 1)},
+           "recurrent_bwd (2 sweeps)": {"ms": round(ms_b, 5), "alg_GBs": round(22 * D * n_th / ms_b / 1e6, 1)}}
+    achieved = alg / ms_step / 1e6
+    return {
+        "value": B * T / ms_step / 1e3,
+        "ms_per_step": ms_step,
+        "roofline": {"bound": "hbm", "kernel": "recurrent fwd+bwd", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "alg_bytes_per_launch": alg},
+        "kernels": per,
+        "valu_frac": round(17 * D * D * n_th / ms_step / 1e9 / FP32_VALU_PEAK_TFLOPS, 4),
+    }
+
+
+def cpu_baseline(B, T, H, D, shift, budget_s=12.0):
+    """The C restatement of recurrent_gla_naive (oracle/), forward + gradients, on one batch element
+    of the workload, repeated until ~budget_s of wall time is spent."""
+    from oracle import gla_oracle as O
+    from oracle import naive_c
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1))
+    Bs = 1
+    h0, g, v, k, q = O.make_inputs(Bs, T, H, D, shift, seed=5)
+    dhT = np.ones_like(h0)
+    dout = np.ones_like(v)
+    naive_c.naive_bwd(h0, g, v, k, q, dhT, dout, dtype=np.float32, nthreads=cores)   # warm-up
+    n, t0 = 0, time.perf_counter()
+    while True:
+        naive_c.naive_bwd(h0, g, v, k, q, dhT, dout, dtype=np.float32, nthreads=cores)
+        n += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s or n >= 50:
+            break
+    return {"value": round(Bs * T * n / el / 1e6, 5), "unit": "Mtokens/s", "cores": cores, "kind": "port",
+            "sample": f"recurrent_gla_naive fwd+bwd (C/OpenMP, fp32 state), B={Bs} of {B}, T={T}, H={H}, D={D}, "
+                      f"{n} repeats in {el:.1f}s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="chunk", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures ONE GPU: every (batch, head) pair is an independent unit, a multi-GPU "
+                 "run is a zero-communication split of them and is not part of this build (--gpus 1 only)")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    kind, B, T, H, D, chunk, shift = WORKLOADS[args.workload]
+    if kind == "chunk":
+        r = bench_chunk(B, T, H, D, chunk, shift, args.steps, args.warmup)
+        metric = "chunk_gla fwd+bwd Mtokens/s (B4,T4096,H6,D128 bf16); % bf16 MFMA peak" \
+            if args.workload == "chunk" else f"chunk_gla fwd+bwd Mtokens/s (B{B},T{T},H{H},D{D} bf16)"
+        wl = f"chunk_gla fwd+bwd B{B} T{T} H{H} D{D} chunk{chunk} bf16, gates log_sigmoid({shift:g}+N(0,1)) fp32"
+    else:
+        r = bench_recurrent(B, T, H, D, shift, args.steps, args.warmup)
+        metric = f"recurrent_gla fwd+bwd Mtokens/s (B{B},T{T},H{H},D{D} bf16); HBM GB/s"
+        wl = f"recurrent_gla fwd+bwd B{B} T{T} H{H} D{D} bf16, gates log_sigmoid({shift:g}+N(0,1)) fp32"
+    line = {
+        "metric": metric, "value": round(r.pop("value"), 4), "unit": "Mtokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(r.pop("ms_per_step"), 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic", "config": {"workload": wl, "B": B, "T": T, "H": H, "D": D, "chunk_size": chunk},
+    }
+    line.update(r)
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(B, T, H, D, shift)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -27,6 +27,8 @@ SIGNATURES = {
     "gla_chunk_bwd_workspace_bytes": (_sz, [_i64] * 6 + [_int]),
     "gla_chunk_fwd": (_int, [_vp] + [_i64] * 6 + [_int] + [_vp] * 9 + [_sz]),
     "gla_chunk_bwd": (_int, [_vp] + [_i64] * 6 + [_int] + [_vp] * 13 + [_sz]),
+    "gla_chunk_fwd_stages": (_int, [_vp, _int] + [_i64] * 6 + [_int] + [_vp] * 9 + [_sz]),
+    "gla_chunk_bwd_stages": (_int, [_vp, _int] + [_i64] * 6 + [_int] + [_vp] * 13 + [_sz]),
 }
 
 _lib = None

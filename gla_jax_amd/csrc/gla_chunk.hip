@@ -78,11 +78,11 @@ extern "C" size_t gla_chunk_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H,
     return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.prod + p.decay + p.states : 0;
 }
 
-extern "C" int gla_chunk_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                             int64_t chunk_size, gla_dtype dtype, const void *hidden_init,
-                             const float *log_fgate, const void *value, const void *key, const void *query,
-                             void *hidden_final, void *out, void *states, void *workspace,
-                             size_t workspace_bytes)
+extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK,
+                                    int64_t DV, int64_t chunk_size, gla_dtype dtype, const void *hidden_init,
+                                    const float *log_fgate, const void *value, const void *key,
+                                    const void *query, void *hidden_final, void *out, void *states,
+                                    void *workspace, size_t workspace_bytes)
 {
     ChunkPlan p;
     int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p);
@@ -103,20 +103,35 @@ extern "C" int gla_chunk_fwd(void *stream, int64_t B, int64_t T, int64_t H, int6
     return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d) -> int {
         typedef decltype(t) E;
         constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value;
-        int e = launch_chunk_outer<E, C_, D_>(st, 0, (int)B, (int)T, (int)H, log_fgate, value, key, prodT, decay);
+        int e = 0;
+        if (stages & 1)
+            e = launch_chunk_outer<E, C_, D_>(st, 0, (int)B, (int)T, (int)H, log_fgate, value, key, prodT, decay);
         if (e) return e;
-        e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 0, hidden_init, prodT, decay, st_buf, hidden_final);
+        if (stages & 2)
+            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 0, hidden_init, prodT, decay, st_buf, hidden_final);
         if (e) return e;
-        return launch_chunk_out<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, st_buf, out);
+        if (stages & 4)
+            e = launch_chunk_out<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, st_buf, out);
+        return e;
     });
 }
 
-extern "C" int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                             int64_t chunk_size, gla_dtype dtype, const float *log_fgate, const void *value,
-                             const void *key, const void *query, const void *states,
-                             const void *dhidden_final, const void *dout, void *dhidden_init,
-                             float *dlog_fgate, void *dvalue, void *dkey, void *dquery, void *workspace,
+extern "C" int gla_chunk_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                             int64_t chunk_size, gla_dtype dtype, const void *hidden_init,
+                             const float *log_fgate, const void *value, const void *key, const void *query,
+                             void *hidden_final, void *out, void *states, void *workspace,
                              size_t workspace_bytes)
+{
+    return gla_chunk_fwd_stages(stream, 7, B, T, H, DK, DV, chunk_size, dtype, hidden_init, log_fgate, value,
+                                key, query, hidden_final, out, states, workspace, workspace_bytes);
+}
+
+extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK,
+                                    int64_t DV, int64_t chunk_size, gla_dtype dtype, const float *log_fgate,
+                                    const void *value, const void *key, const void *query, const void *states,
+                                    const void *dhidden_final, const void *dout, void *dhidden_init,
+                                    float *dlog_fgate, void *dvalue, void *dkey, void *dquery,
+                                    void *workspace, size_t workspace_bytes)
 {
     ChunkPlan p;
     int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p);
@@ -138,11 +153,28 @@ extern "C" int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int6
     return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d) -> int {
         typedef decltype(t) E;
         constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value;
-        int e = launch_chunk_outer<E, C_, D_>(st, 1, (int)B, (int)T, (int)H, log_fgate, dout, query, prodT, decay);
+        int e = 0;
+        if (stages & 1)
+            e = launch_chunk_outer<E, C_, D_>(st, 1, (int)B, (int)T, (int)H, log_fgate, dout, query, prodT, decay);
         if (e) return e;
-        e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 1, dhidden_final, prodT, decay, dstates, dhidden_init);
+        if (stages & 2)
+            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 1, dhidden_final, prodT, decay, dstates, dhidden_init);
         if (e) return e;
-        return launch_chunk_grad<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,
-                                            states, dstates, decay, dlog_fgate, dvalue, dkey, dquery);
+        if (stages & 4)
+            e = launch_chunk_grad<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,
+                                             states, dstates, decay, dlog_fgate, dvalue, dkey, dquery);
+        return e;
     });
+}
+
+extern "C" int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                             int64_t chunk_size, gla_dtype dtype, const float *log_fgate, const void *value,
+                             const void *key, const void *query, const void *states,
+                             const void *dhidden_final, const void *dout, void *dhidden_init,
+                             float *dlog_fgate, void *dvalue, void *dkey, void *dquery, void *workspace,
+                             size_t workspace_bytes)
+{
+    return gla_chunk_bwd_stages(stream, 7, B, T, H, DK, DV, chunk_size, dtype, log_fgate, value, key, query,
+                                states, dhidden_final, dout, dhidden_init, dlog_fgate, dvalue, dkey, dquery,
+                                workspace, workspace_bytes);
 }

@@ -18,6 +18,13 @@
 //   d(log-gate cumsum) per token is q*dq - k*dk (the anchors cancel, gla.py:1078-1087); dlog_fgate is
 //     its reverse cumsum inside the chunk plus the chunk-level term of gla.py:782.
 // All sums that feed dlog_fgate stay in fp32 registers (gla.py:1073-1087 asks for fp32 there).
+//
+// Register plan.  Everything indexed by (token, feature) is needed only 32 features at a time, while the
+// 16x16 score blocks do not depend on the feature at all.  So each role first computes and caches
+// its score blocks (packed MFMA operands, 2 registers each), then walks the head dimension in slices
+// of 32 features: levels, chain, epilogue, store.  What has to survive from the first role to the
+// second (the sub-block part of dk, the query-side gate gradient) is parked in the token's rows of
+// outputs that are written last, and read back (L2 hits) by the same lane.
 #include "gla_chunk_common.hpp"
 #include "gla_chunk_kernels.hpp"
 
@@ -33,6 +40,15 @@ __device__ __forceinline__ f32x8 join4(f32x4 lo, f32x4 hi)
 #pragma unroll
     for (int e = 0; e < 4; ++e) { r.v[e] = lo[e]; r.v[4 + e] = hi[e]; }
     return r;
+}
+
+// Hides a pointer's provenance from the optimiser: loads through the result are not merged with
+// earlier loads of (or forwarded from earlier stores to) the same address, so a value can be dropped
+// from registers and fetched again (an L2 hit) where it is needed next.
+template <typename P> __device__ __forceinline__ P *refetch(P *ptr)
+{
+    asm volatile("" : "+v"(ptr));
+    return ptr;
 }
 
 // inclusive suffix sum over the 16 token rows of the wave (lane r receives sum over rows >= r)
@@ -52,144 +68,112 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const T *__restrict__ dstates, const float *__restrict__ decay, float *__restrict__ dg,
     T *__restrict__ dv, T *__restrict__ dk, T *__restrict__ dq, int T_len, int H)
 {
-    constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16;
+    constexpr int NB = C / 16, KS = D / 32, NV = D / 4;
     constexpr int LS = TileGeom<T, D>::kStride;
-    constexpr int TR = C > D ? C : D;   // rows of one LDS tile
+    constexpr int XS = 32 + 16 / (int)sizeof(T);   // row stride of the per-wave slice scratch
+    constexpr int TR = C > D ? C : D;              // rows of one LDS tile
     typedef typename FragTypes<T>::d8 D8;
+    typedef typename FragTypes<T>::t4 T4;
     extern __shared__ __align__(16) unsigned char smem[];
-    T *tile0 = reinterpret_cast<T *>(smem);
-    T *tile1 = tile0 + TR * LS;
-    T *tile2 = tile1 + TR * LS;
-    T *xs = tile2 + TR * LS;                                   // [NB][16][LS] per-wave scratch
-    float *rtab = reinterpret_cast<float *>(xs + NB * 16 * LS);   // [NB][D] e^{tau_m}
-    float *dltab = rtab + NB * D;                              // [NB][D] sub-block sums of q*dq - k*dk
-    float *lbar = dltab + NB * D;                              // [D] chunk-level gate gradient
+    T *tile0 = reinterpret_cast<T *>(smem);        // value, later dout                  [token][dv]
+    T *tile1 = tile0 + TR * LS;                    // k e^{tau_J - l_j}                  [token][dk]
+    T *tile2 = tile1 + TR * LS;                    // S_n, later dS'                     [dv][dk]
+    T *tile3 = tile2 + TR * LS;                    // q e^{l_i}                          [token][dk]
+    T *xs = tile3 + TR * LS;                       // [NB][16][XS] per-wave scratch
+    float *rtab = reinterpret_cast<float *>(xs + NB * 16 * XS);   // [NB][D] e^{tau_m}
+    float *dltab = rtab + NB * D;                  // [NB][D] sub-block sums of the gate-cumsum gradient
+    float *lbar = dltab + NB * D;                  // [D] chunk-level gate gradient
 
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: scalar branches on it
     const int r = lane & 15, c = lane >> 4;
     const int n = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int N = T_len / C;
     const int64_t tok = (int64_t)b * T_len + (int64_t)n * C + 16 * w + r;
     const int64_t rowoff = (tok * H + h) * D;
     const int64_t bhn = ((int64_t)b * H + h) * N + n;
-    T *xw = xs + w * 16 * LS;
+    const TrLane<T> L = make_tr_lane<T>(LS);
+    const TrLane<T> Lx = make_tr_lane<T>(XS);
+    const int wrow = 16 * w * LS + L.nat;          // this lane's row of a [token][feature] tile
+    T *xw = xs + w * 16 * XS;                      // [16][XS]: one 32-feature slice of the wave's rows
 
-    float p[NV], s[NV];
-    D8 qf[KS], kf[KS], vf[KS], dof[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        const int d0 = 32 * ks + 8 * c;
-        f32x8 gg = ld8(g + rowoff + d0);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
-        qf[ks] = ld8(q + rowoff + d0);
-        kf[ks] = ld8(k + rowoff + d0);
-        vf[ks] = ld8(v + rowoff + d0);
-        dof[ks] = ld8(dout + rowoff + d0);
-    }
-    if (threadIdx.x < D) lbar[threadIdx.x] = 0.f;
-
-    // ---- the wave's own sub-block ----------------------------------------------------------------
-    // dAn[e] = dA[i = 4c+e][j = r],  dAt[e] = dA[i = r][j = 4c+e]   (dA = dO V^T)
-    f32x4 dAn = {0.f, 0.f, 0.f, 0.f}, dAt = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        dAn = mma_d(dof[ks], vf[ks], dAn);
-        dAt = mma_d(vf[ks], dof[ks], dAt);
-    }
+    D8 dof[KS];
     f32x4 Aown = {0.f, 0.f, 0.f, 0.f};   // scores A[i = 4c+e][j = r] of the own sub-block
-    float dqa[NV], dka[NV];             // sub-block parts of dq, dk (row layout)
-    // Gradient w.r.t. the gate cumsum L of this row.  Every term dA_ij * q~_i * k~_j enters row i with +
-    // and row j with -; both sides are formed from the SAME rounded operands (the values the MFMAs
-    // consume), so the two copies cancel exactly in the reverse cumsum (gla.py:1077-1087 asks for this).
-    float dlm[NV];
-#pragma unroll
-    for (int i = 0; i < NV; ++i) { dqa[i] = 0.f; dka[i] = 0.f; dlm[i] = 0.f; }
-
-    auto level = [&](auto hc) {
-        constexpr int h_ = decltype(hc)::value;
-        const bool upper = (r & h_) != 0;
-        float fac[NV];
-        D8 Xf[KS];
-        f32x4 G = {0.f, 0.f, 0.f, 0.f};
+    T4 symb[4];                          // per level: masked (dA + dA^T) of the own sub-block, MFMA operand
+    float dd = 0.f;                      // dA_ii of this lane's row
+    {
+        float p[NV], s[NV];
+        D8 vf[KS], qf[KS], kf[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            float a[8], bq[8], x[8];
+            const int d0 = 32 * ks + 8 * c;
+            f32x8 gg = ld8(g + rowoff + d0);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
+            qf[ks] = ld8(q + rowoff + d0);
+            kf[ks] = ld8(k + rowoff + d0);
+            vf[ks] = ld8(v + rowoff + d0);
+            dof[ks] = ld8(dout + rowoff + d0);
+            st8(tile0 + wrow + 32 * ks, vf[ks]);
+        }
+        if (threadIdx.x < D) lbar[threadIdx.x] = 0.f;
+
+        // dAn[e] = dA[i = 4c+e][j = r],  dAt[e] = dA[i = r][j = 4c+e]   (dA = dO V^T), own sub-block
+        f32x4 dAn = {0.f, 0.f, 0.f, 0.f}, dAt = {0.f, 0.f, 0.f, 0.f};
+        float dot = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            dAn = mma_d(dof[ks], vf[ks], dAn);
+            dAt = mma_d(vf[ks], dof[ks], dAt);
+            float a[8], bq[8];
             unpack8(qf[ks], a);
             unpack8(kf[ks], bq);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                fac[8 * ks + e] = fast_exp2(upper ? p[8 * ks + e] : s[8 * ks + e]);
-                x[e] = (upper ? a[e] : bq[e]) * fac[8 * ks + e];
-            }
-            Xf[ks] = pack8<T>(x);
-            G = mma_d(Xf[ks], Xf[ks], G);
-            st8(xw + r * LS + 32 * ks + 8 * c, Xf[ks]);
+            for (int e = 0; e < 8; ++e) dot += a[e] * bq[e];
         }
-        f32x4 sym;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int o = 4 * c + e;                       // the other row
-            const bool same = (o ^ r) < 2 * h_;
-            const bool o_up = (o & h_) != 0;
-            Aown[e] += (same && o_up && !upper) ? G[e] : 0.f;
-            sym[e] = (same && upper && !o_up) ? dAt[e] : ((same && o_up && !upper) ? dAn[e] : 0.f);
-        }
-        __syncthreads();
-        auto b4 = pack4<T>(sym);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            float xr[8];
-            unpack8(Xf[ks], xr);
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                const int t = 2 * ks + tt;
-                const PiCols pc = pi_cols(t);
-                f32x4 dx = {0.f, 0.f, 0.f, 0.f};
-                dx = mma_t(lds_tr4(xw, LS, 4 * c, pc.seg, pc.own), b4, dx);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float z = dx[e] * fac[4 * t + e];
-                    dqa[4 * t + e] += upper ? z : 0.f;
-                    dka[4 * t + e] += upper ? 0.f : z;
-                    const float y = dx[e] * xr[4 * tt + e];
-                    dlm[4 * t + e] += upper ? y : -y;
-                }
-            }
-        }
-        hier_step<h_>(p, s, upper);
-        __syncthreads();
-    };
-    level(std::integral_constant<int, 1>{});
-    level(std::integral_constant<int, 2>{});
-    level(std::integral_constant<int, 4>{});
-    level(std::integral_constant<int, 8>{});
-
-    // diagonal entries, rescaled key tile, table of e^{tau}
-    {
-        float dd = 0.f, dot = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) dd += (4 * c + e == r) ? dAt[e] : 0.f;
         dd = reduce_over_cgroups(dd);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            float a[8], bq[8], kh[8];
-            unpack8(qf[ks], a);
-            unpack8(kf[ks], bq);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                dot += a[e] * bq[e];
-                dqa[8 * ks + e] += dd * bq[e];
-                dka[8 * ks + e] += dd * a[e];
-                kh[e] = bq[e] * fast_exp2(s[8 * ks + e]);
-            }
-            const int d0 = 32 * ks + 8 * c;
-            st8(tile1 + (16 * w + r) * LS + d0, pack8<T>(kh));
-            st8(tile0 + (16 * w + r) * LS + d0, vf[ks]);
-        }
         dot = reduce_over_cgroups(dot);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) Aown[e] += (4 * c + e == r) ? dot : 0.f;
+        for (int e = 0; e < 4; ++e) Aown[e] = (4 * c + e == r) ? dot : 0.f;   // A_ii = q_i.k_i (gla.py:983)
+
+        // Pass 1 over the dyadic levels, full head dimension: the mixed tile X of every level -> the
+        // level's score blocks (they contract over all features), and the gate prefix/suffix sums.
+        auto level_scores = [&](auto hc, auto lc) {
+            constexpr int h_ = decltype(hc)::value, L_ = decltype(lc)::value;
+            const bool upper = (r & h_) != 0;
+            f32x4 G = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                float a[8], bq[8], x[8];
+                unpack8(qf[ks], a);
+                unpack8(kf[ks], bq);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    x[e] = (upper ? a[e] : bq[e]) * fast_exp2(upper ? p[8 * ks + e] : s[8 * ks + e]);
+                D8 X = pack8<T>(x);
+                G = mma_d(X, X, G);
+            }
+            f32x4 sym;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int o = 4 * c + e;                       // the other row
+                const bool same = (o ^ r) < 2 * h_;
+                const bool o_up = (o & h_) != 0;
+                Aown[e] += (same && o_up && !upper) ? G[e] : 0.f;
+                sym[e] = (same && upper && !o_up) ? dAt[e] : ((same && o_up && !upper) ? dAn[e] : 0.f);
+            }
+            symb[L_] = pack4<T>(sym);
+            hier_step<h_>(p, s, upper);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        level_scores(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+        level_scores(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
+        level_scores(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
+        level_scores(std::integral_constant<int, 8>{}, std::integral_constant<int, 3>{});
+
+        // p = l_i, s = tau - l_i (log2 units): table of e^{tau}, rescaled key and query tiles
         if (r == 0) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -199,6 +183,19 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 st8(rtab + w * D + 32 * ks + 8 * c, t);
             }
         }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            float a[8], bq[8];
+            unpack8(qf[ks], a);
+            unpack8(kf[ks], bq);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                a[e] *= fast_exp2(p[8 * ks + e]);
+                bq[e] *= fast_exp2(s[8 * ks + e]);
+            }
+            st8(tile3 + wrow + 32 * ks, pack8<T>(a));
+            st8(tile1 + wrow + 32 * ks, pack8<T>(bq));
+        }
         const T *sp = states + bhn * D * D;
         for (int idx = threadIdx.x; idx < D * D / 8; idx += C * 4) {
             const int row = idx / (D / 8), c8 = (idx % (D / 8)) * 8;
@@ -207,73 +204,143 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     }
     __syncthreads();
 
-    // ---- row-owner role: dq ----------------------------------------------------------------------
-    {
-        f32x4 acc[NT];
+    // ---- row-owner role ----------------------------------------------------------------------------
+    // score blocks dA^T of the earlier sub-blocks: dAT_J[j][i] = v_j . dO_i  (J < w)
+    T4 dATc[NB];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int J = 0; J < NB - 1; ++J) {
+        dATc[J] = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
+        if (J < w) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
+            for (int ks = 0; ks < KS; ++ks) a = mma_d(ld8(tile0 + L.nat + 16 * J * LS + 32 * ks), dof[ks], a);
+            dATc[J] = pack4<T>(a);
+        }
+    }
+    dATc[NB - 1] = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
+    __builtin_amdgcn_sched_barrier(0);
+
+    // Gradient w.r.t. the gate cumsum L of a row, "dL".  Every term dA_ij * q~_i * k~_j enters row i with +
+    // and row j with -; both copies are formed from the SAME rounded operands (the values the MFMAs
+    // consume), so they cancel exactly in the reverse cumsum (gla.py:1077-1087 asks for this).
+    //
+    // The head dimension is walked in slices of 32 features by a real (not unrolled) loop, so that only
+    // one slice's temporaries are live.  What has to survive from this loop to the column-owner loop
+    // is parked in the token's rows of the outputs that are written last: the sub-block part of dk in the
+    // dlog_fgate row (fp32), the query-side dL in the dk and dv rows (together D fp32 values).
+#pragma unroll 1
+    for (int ks = 0; ks < KS; ++ks) {
+        const int fo = 32 * ks;
+        float p8[8], s8[8], a[8], bq[8], dq8[8], dk8[8], dl8[8];
+        {
+            f32x8 gg = ld8(refetch(g + rowoff) + fo + 8 * c);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                const PiCols pc = pi_cols(t);
-                auto a = join4(lds_tr4(tile2, LS, 32 * ks + 8 * c, pc.seg, pc.own),
-                               lds_tr4(tile2, LS, 32 * ks + 8 * c + 4, pc.seg, pc.own));
-                acc[t] = mma_d(a, dof[ks], acc[t]);
+            for (int e = 0; e < 8; ++e) { p8[e] = gg.v[e] * kLog2e; s8[e] = 0.f; }
+            unpack8(ld8(refetch(q + rowoff) + fo + 8 * c), a);
+            unpack8(ld8(refetch(k + rowoff) + fo + 8 * c), bq);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            dq8[e] = dd * bq[e];         // diagonal term dA_ii q_i k_i: no gate gradient (gla.py:1181-1185)
+            dk8[e] = dd * a[e];
+            dl8[e] = 0.f;
+        }
+        // A level of the dyadic recursion restricted to the slice: rebuilds the slice of X, dX = (M + M^T) X
+        // by one MFMA per 16 features, and adds its share to the sub-block parts of dq / dk / dL.  The
+        // per-wave scratch is written and read by the same wave only; LDS executes one wave's accesses
+        // in order, so a compiler-level fence is all the ordering that is needed.
+        auto slice_level = [&](auto hc, auto lc) {
+            constexpr int h_ = decltype(hc)::value, L_ = decltype(lc)::value;
+            const bool upper = (r & h_) != 0;
+            float fac[8], x[8], xr[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                fac[e] = fast_exp2(upper ? p8[e] : s8[e]);
+                x[e] = (upper ? a[e] : bq[e]) * fac[e];
+            }
+            D8 X = pack8<T>(x);
+            unpack8(X, xr);
+            st8(xw + Lx.nat, X);
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                f32x4 dx = {0.f, 0.f, 0.f, 0.f};
+                dx = mma_t(lds_tr4(xw + Lx.k4 + 4 * tt, XS), symb[L_], dx);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float z = dx[e] * fac[4 * tt + e];
+                    const float y = dx[e] * xr[4 * tt + e];
+                    dq8[4 * tt + e] += upper ? z : 0.f;
+                    dk8[4 * tt + e] += upper ? 0.f : z;
+                    dl8[4 * tt + e] += upper ? y : -y;
+                }
+            }
+            asm volatile("" ::: "memory");
+            hier_step<h_>(p8, s8, upper);
+        };
+        slice_level(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+        slice_level(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
+        slice_level(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
+        slice_level(std::integral_constant<int, 8>{}, std::integral_constant<int, 3>{});
+        {
+            f32x8 pk;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pk.v[e] = dk8[e];
+            st8(dg + rowoff + fo + 8 * c, pk);               // parked until the dk epilogue
+        }
+
+        // dq chain of the slice: state term first, then the earlier sub-blocks in ascending order
+        f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+        for (int k2 = 0; k2 < KS; ++k2) {
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                const T *bp = tile2 + L.k8 + fo + 4 * tt + 32 * k2 * LS;
+                acc[tt] = mma_d(join4(lds_tr4(bp, LS), lds_tr4(bp + 4 * LS, LS)), dof[k2], acc[tt]);
             }
         }
 #pragma unroll
         for (int J = 0; J < NB - 1; ++J) {
             if (J < w) {
-                f32x4 dAT = {0.f, 0.f, 0.f, 0.f};
+                f32x8 rr = ld8(rtab + J * D + fo + 8 * c);
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    f32x8 rr = ld8(rtab + J * D + 32 * ks + 8 * c);
+                for (int tt = 0; tt < 2; ++tt) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        acc[2 * ks][e] *= rr.v[e];
-                        acc[2 * ks + 1][e] *= rr.v[4 + e];
-                    }
-                    dAT = mma_d(ld8(tile0 + (16 * J + r) * LS + 32 * ks + 8 * c), dof[ks], dAT);
-                }
-                auto b4 = pack4<T>(dAT);
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const PiCols pc = pi_cols(t);
-                    acc[t] = mma_t(lds_tr4(tile1, LS, 16 * J + 4 * c, pc.seg, pc.own), b4, acc[t]);
+                    for (int e = 0; e < 4; ++e) acc[tt][e] *= rr.v[4 * tt + e];
+                    acc[tt] = mma_t(lds_tr4(tile1 + L.k4 + fo + 4 * tt + 16 * J * LS, LS), dATc[J], acc[tt]);
                 }
             }
         }
+        {
+            float o[8], qe[8], qr[8];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            float a[8], o[8], qr[8];
-            unpack8(qf[ks], a);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) a[e] *= fast_exp2(p[8 * ks + e]);
-            unpack8(pack8<T>(a), qr);                    // q e^{l} as the MFMAs of the key side see it
+            for (int e = 0; e < 8; ++e) qe[e] = a[e] * fast_exp2(p8[e]);
+            unpack8(pack8<T>(qe), qr);                   // q e^{l} as the MFMAs of the key side see it
+            f32x4 lo, hi;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float hacc = e < 4 ? acc[2 * ks][e] : acc[2 * ks + 1][e - 4];
-                o[e] = fast_exp2(p[8 * ks + e]) * hacc + dqa[8 * ks + e];
-                dlm[8 * ks + e] += qr[e] * hacc;
+                const float hacc = acc[e >> 2][e & 3];
+                o[e] = fast_exp2(p8[e]) * hacc + dq8[e];
+                const float dl = dl8[e] + qr[e] * hacc;
+                if (e < 4) lo[e] = dl; else hi[e - 4] = dl;
             }
-            st8(dq + rowoff + 32 * ks + 8 * c, pack8<T>(o));
+            st8(dq + rowoff + fo + 8 * c, pack8<T>(o));
+            // query-side dL, parked: 8 fp32 = the slice's 8 elements of the dk row + of the dv row
+            if constexpr (sizeof(T) == 2) {
+                *reinterpret_cast<f32x4 *>(dk + rowoff + fo + 8 * c) = lo;
+                *reinterpret_cast<f32x4 *>(dv + rowoff + fo + 8 * c) = hi;
+            } else {
+                f32x8 both = join4(lo, hi);
+                st8(reinterpret_cast<float *>(dk + rowoff + fo + 8 * c), both);
+            }
         }
     }
     __syncthreads();
 
-    // ---- second set of tiles: dO, q e^{l}, dS'^T; chunk-level term sum_v S*dS' ---------------------
+    // ---- second set of tiles: dO, dS'^T; chunk-level term sum_v S*dS' ------------------------------
     {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            float a[8];
-            unpack8(qf[ks], a);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) a[e] *= fast_exp2(p[8 * ks + e]);
-            const int d0 = 32 * ks + 8 * c;
-            st8(tile1 + (16 * w + r) * LS + d0, pack8<T>(a));
-            st8(tile0 + (16 * w + r) * LS + d0, dof[ks]);
-        }
+        for (int ks = 0; ks < KS; ++ks) st8(tile0 + wrow + 32 * ks, dof[ks]);
         const T *dsp = dstates + bhn * D * D;
         float part[8];
 #pragma unroll
@@ -295,142 +362,153 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     }
     __syncthreads();
 
-    // ---- column-owner role: scores, dv ------------------------------------------------------------
-    float kch[NV];   // k e^{tau_J - l_j}, walked up to k e^{L_end - L_j}
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        float bq[8];
-        unpack8(kf[ks], bq);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) kch[8 * ks + e] = bq[e] * fast_exp2(s[8 * ks + e]);
-    }
+    // ---- column-owner role -------------------------------------------------------------------------
+    // score blocks of the later sub-blocks: A_IJ (needs the key side walked up by r_I) and dA_IJ
+    T4 Ac[NB], dAc[NB];
+    D8 Kt[KS], vf[KS];                   // k e^{L_end - L_j} as MFMA operand; value rows
     {
-        f32x4 Ab[NB];
+        float kch[NV];
+        const T *vp = refetch(v + rowoff);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            vf[ks] = ld8(vp + 32 * ks + 8 * c);
+            unpack8(ld8(tile1 + wrow + 32 * ks), kch + 8 * ks);
+        }
 #pragma unroll
         for (int I = 1; I < NB; ++I) {
-            Ab[I] = f32x4{0.f, 0.f, 0.f, 0.f};
+            Ac[I] = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
+            dAc[I] = Ac[I];
             if (I > w) {
+                f32x4 a = {0.f, 0.f, 0.f, 0.f}, da = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    Ab[I] = mma_d(ld8(tile1 + (16 * I + r) * LS + 32 * ks + 8 * c), pack8<T>(kch + 8 * ks), Ab[I]);
+                    a = mma_d(ld8(tile3 + L.nat + 16 * I * LS + 32 * ks), pack8<T>(kch + 8 * ks), a);
+                    da = mma_d(ld8(tile0 + L.nat + 16 * I * LS + 32 * ks), vf[ks], da);
                     f32x8 rr = ld8(rtab + I * D + 32 * ks + 8 * c);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) kch[8 * ks + e] *= rr.v[e];
                 }
+                Ac[I] = pack4<T>(a);
+                dAc[I] = pack4<T>(da);
             }
         }
-        Ab[0] = f32x4{0.f, 0.f, 0.f, 0.f};
-        f32x4 acc[NT];
+        Ac[0] = pack4<T>(Aown);
+        dAc[0] = Ac[0];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            D8 kb = pack8<T>(kch + 8 * ks);
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-                acc[t] = mma_d(ld8(tile2 + pi_cols(t).own * LS + 32 * ks + 8 * c), kb, acc[t]);
-        }
-#pragma unroll
-        for (int I = 0; I < NB; ++I) {
-            if (I >= w) {
-                auto b4 = pack4<T>(I == w ? Aown : Ab[I]);
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const PiCols pc = pi_cols(t);
-                    acc[t] = mma_t(lds_tr4(tile0, LS, 16 * I + 4 * c, pc.seg, pc.own), b4, acc[t]);
-                }
-            }
-        }
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            float o[8];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { o[e] = acc[2 * ks][e]; o[4 + e] = acc[2 * ks + 1][e]; }
-            st8(dv + rowoff + 32 * ks + 8 * c, pack8<T>(o));
-        }
+        for (int ks = 0; ks < KS; ++ks) Kt[ks] = pack8<T>(kch + 8 * ks);
     }
 
-    // ---- column-owner role: dk, then dlog_fgate ----------------------------------------------------
-    {
-        f32x4 acc[NT];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-#pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                const PiCols pc = pi_cols(t);
-                auto a = join4(lds_tr4(tile2, LS, 32 * ks + 8 * c, pc.seg, pc.own),
-                               lds_tr4(tile2, LS, 32 * ks + 8 * c + 4, pc.seg, pc.own));
-                acc[t] = mma_d(a, vf[ks], acc[t]);
-            }
+#pragma unroll 1
+    for (int ks = 0; ks < KS; ++ks) {
+        const int fo = 32 * ks;
+        // what the row-owner loop parked for this slice (read before the rows are overwritten below)
+        f32x8 dlq;
+        if constexpr (sizeof(T) == 2) {
+            dlq = join4(*reinterpret_cast<const f32x4 *>(refetch(dk + rowoff) + fo + 8 * c),
+                        *reinterpret_cast<const f32x4 *>(refetch(dv + rowoff) + fo + 8 * c));
+        } else {
+            dlq = ld8(reinterpret_cast<const float *>(refetch(dk + rowoff) + fo + 8 * c));
         }
-        // chunk-level gate gradient, key part: sum_j (k e^{L_end - L_j}) * (V dS'^T)_j
+        // dv slice
+        {
+            f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
+            for (int k2 = 0; k2 < KS; ++k2) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float z = reduce_over_rows(kch[4 * t + e] * acc[t][e]);
-                if (r == 0) atomicAdd(lbar + 32 * (t >> 1) + 8 * c + 4 * (t & 1) + e, z);
+                for (int tt = 0; tt < 2; ++tt)
+                    acc[tt] = mma_d(ld8(tile2 + L.own + (fo + 4 * tt) * LS + 32 * k2), Kt[k2], acc[tt]);
             }
+#pragma unroll
+            for (int I = 0; I < NB; ++I) {
+                if (I >= w) {
+                    const T4 b4 = I == w ? Ac[0] : Ac[I];
+#pragma unroll
+                    for (int tt = 0; tt < 2; ++tt)
+                        acc[tt] = mma_t(lds_tr4(tile0 + L.k4 + fo + 4 * tt + 16 * I * LS, LS), b4, acc[tt]);
+                }
+            }
+            float o[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
+            st8(dv + rowoff + fo + 8 * c, pack8<T>(o));
         }
+        // dk slice
+        {
+            f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-        for (int I = NB - 1; I >= 1; --I) {
-            if (I > w) {
-                f32x4 dAI = {0.f, 0.f, 0.f, 0.f};
+            for (int k2 = 0; k2 < KS; ++k2) {
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    f32x8 rr = ld8(rtab + I * D + 32 * ks + 8 * c);
+                for (int tt = 0; tt < 2; ++tt) {
+                    const T *bp = tile2 + L.k8 + fo + 4 * tt + 32 * k2 * LS;
+                    acc[tt] = mma_d(join4(lds_tr4(bp, LS), lds_tr4(bp + 4 * LS, LS)), vf[k2], acc[tt]);
+                }
+            }
+            float kr[8];
+            unpack8(ld8(tile1 + wrow + fo), kr);           // k e^{tau-l} as the MFMAs saw it
+            // chunk-level gate gradient, key part: sum_j (k e^{L_end - L_j}) * (V dS'^T)_j, with
+            // k e^{L_end - L_j} = (k e^{tau - l_j}) * prod_{m > w} r_m
+            {
+                float sig[8];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        acc[2 * ks][e] *= rr.v[e];
-                        acc[2 * ks + 1][e] *= rr.v[4 + e];
+                for (int e = 0; e < 8; ++e) sig[e] = 1.f;
+                for (int m = w + 1; m < NB; ++m) {
+                    f32x8 rr = ld8(rtab + m * D + fo + 8 * c);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sig[e] *= rr.v[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float z = reduce_over_rows(kr[e] * acc[e >> 2][e & 3]) * sig[e];
+                    if (r == 0) atomicAdd(lbar + fo + 8 * c + e, z);
+                }
+            }
+#pragma unroll
+            for (int I = NB - 1; I >= 1; --I) {
+                if (I > w) {
+                    f32x8 rr = ld8(rtab + I * D + fo + 8 * c);
+#pragma unroll
+                    for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[tt][e] *= rr.v[4 * tt + e];
+                        acc[tt] = mma_t(lds_tr4(tile3 + L.k4 + fo + 4 * tt + 16 * I * LS, LS), dAc[I], acc[tt]);
                     }
-                    dAI = mma_d(ld8(tile0 + (16 * I + r) * LS + 32 * ks + 8 * c), vf[ks], dAI);
-                }
-                auto b4 = pack4<T>(dAI);
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const PiCols pc = pi_cols(t);
-                    acc[t] = mma_t(lds_tr4(tile1, LS, 16 * I + 4 * c, pc.seg, pc.own), b4, acc[t]);
                 }
             }
-        }
+            // epilogue: e^{tau - l} of the slice is rebuilt from the gates (4 prefix/suffix steps)
+            float p8[8], s8[8], o[8];
+            {
+                f32x8 gg = ld8(refetch(g + rowoff) + fo + 8 * c);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            float bq[8], o[8], kr[8];
-            unpack8(kf[ks], bq);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) bq[e] *= fast_exp2(s[8 * ks + e]);
-            unpack8(pack8<T>(bq), kr);                   // k e^{tau-l} as the MFMAs of the query side see it
+                for (int e = 0; e < 8; ++e) { p8[e] = gg.v[e] * kLog2e; s8[e] = 0.f; }
+            }
+            hier_step<1>(p8, s8, (r & 1) != 0);
+            hier_step<2>(p8, s8, (r & 2) != 0);
+            hier_step<4>(p8, s8, (r & 4) != 0);
+            hier_step<8>(p8, s8, (r & 8) != 0);
+            f32x8 parked = ld8(refetch(dg + rowoff) + fo + 8 * c);
+            f32x8 sfx;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float hacc = e < 4 ? acc[2 * ks][e] : acc[2 * ks + 1][e - 4];
-                o[e] = fast_exp2(s[8 * ks + e]) * hacc + dka[8 * ks + e];
-                dlm[8 * ks + e] -= kr[e] * hacc;
+                const float hacc = acc[e >> 2][e & 3];
+                o[e] = fast_exp2(s8[e]) * hacc + parked.v[e];
+                // dL of the row, then its reverse cumsum inside the sub-block (gla.py:616-617)
+                sfx.v[e] = suffix_sum_rows(dlq.v[e] - kr[e] * hacc);
             }
-            st8(dk + rowoff + 32 * ks + 8 * c, pack8<T>(o));
-        }
-    }
-    // reverse cumsum inside the chunk (gla.py:616-617)
-#pragma unroll
-    for (int i = 0; i < NV; ++i) dlm[i] = suffix_sum_rows(dlm[i]);
-    if (r == 0) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            f32x8 t;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) t.v[e] = dlm[8 * ks + e];
-            st8(dltab + w * D + 32 * ks + 8 * c, t);
+            st8(dk + rowoff + fo + 8 * c, pack8<T>(o));
+            st8(dg + rowoff + fo + 8 * c, sfx);               // parked until the other sub-blocks' totals are known
+            if (r == 0) st8(dltab + w * D + fo + 8 * c, sfx);
         }
     }
     __syncthreads();
+
+    // ---- dlog_fgate = reverse cumsum over the whole chunk + the chunk-level term (gla.py:782) ------------
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const int d0 = 32 * ks + 8 * c;
         f32x8 o = ld8(lbar + d0);
+        f32x8 own = ld8(refetch(dg + rowoff) + d0);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o.v[e] += dlm[8 * ks + e];
+        for (int e = 0; e < 8; ++e) o.v[e] += own.v[e];
         for (int m = w + 1; m < NB; ++m) {
             f32x8 t = ld8(dltab + m * D + d0);
 #pragma unroll
@@ -446,8 +524,10 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
                       const float *decay, float *dg, void *dv, void *dk, void *dq)
 {
     constexpr int LS = TileGeom<T, D>::kStride;
+    constexpr int XS = 32 + 16 / (int)sizeof(T);
     constexpr int TR = C > D ? C : D, NB = C / 16;
-    const size_t lds = (size_t)(3 * TR + NB * 16) * LS * sizeof(T) + (size_t)(2 * NB + 1) * D * sizeof(float);
+    const size_t lds = ((size_t)4 * TR * LS + (size_t)NB * 16 * XS) * sizeof(T) +
+                       (size_t)(2 * NB + 1) * D * sizeof(float);
     auto kern = chunk_grad_kernel<T, C, D>;
     if (int e = allow_lds((const void *)kern, lds)) return e;
     dim3 grid(T_len / C, H, B), block(C * 4);

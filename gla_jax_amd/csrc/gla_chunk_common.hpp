@@ -118,49 +118,66 @@ template <typename T, int D> struct TileGeom {
     static constexpr int kStride = D + 16 / (int)sizeof(T);
 };
 
-// Transposing LDS read: for a natural [row][col] tile, returns to lane (i = lane % 16) the four
-// elements tile[krow0 + 0..3][colbase(i / 4) + i % 4].  On bf16 this is one ds_read_b64_tr_b16: the
-// 16 lanes of a group each fetch 4 consecutive columns (lane j of the group: row krow0 + j/4,
-// columns colseg .. colseg+3 where colseg is THAT lane's colbase(j % 4)), and the hardware hands lane i
-// column i%4 of the lanes i/4, i/4+4, i/4+8, i/4+12.  `colseg` is therefore colbase(lane%4) and
-// `colown` is colbase((lane%16)/4) + lane%4, both computed by the caller.
-__device__ __forceinline__ bf16x4 lds_tr4(const __bf16 *tile, int stride, int krow0, int colseg, int colown)
+// Transposing LDS read.  For a natural [row][col] tile and a 4-row band starting at row k0, lane
+// i = lane % 16 of every 16-lane group receives tile[k0 + 0..3][colbase(i / 4) + i % 4].  On bf16 this is
+// one ds_read_b64_tr_b16: lane j of the group fetches 4 consecutive columns (8 bytes) of row
+// k0 + j/4 starting at ITS colbase(j % 4), and the hardware hands lane i column i%4 of the lanes i/4,
+// i/4+4, i/4+8, i/4+12.  With the feature permutation pi, colbase(m) = 32*(t/2) + 8*m + 4*(t%2).
+//
+// All addresses are split into a per-lane part, computed once per kernel (TrLane), and a compile-time
+// part that folds into the instruction's immediate offset, so a kernel keeps a handful of address
+// registers instead of one per (tile, sub-block, feature tile).
+template <typename T> struct TrLane {
+    int nat;   // natural reads:   row r,            features 8c..8c+7          -> r*S + 8c
+    int k4;    // transposed read: rows 4c + ...,    feature block (r>>2 | r&3)
+    int k8;    // transposed read: rows 8c + ...  (contractions over 32 rows, two reads 4 rows apart)
+    int own;   // natural read of the row pi(., m = r): (8*(r>>2) + (r&3))*S + 8c
+};
+template <typename T> __device__ __forceinline__ TrLane<T> make_tr_lane(int stride)
 {
-    (void)colown;
-    const int r = threadIdx.x & 15;
-    const __bf16 *p = tile + (krow0 + (r >> 2)) * stride + colseg;
+    const int lane = threadIdx.x & 63, r = lane & 15, c = lane >> 4;
+    TrLane<T> t;
+    t.nat = r * stride + 8 * c;
+    t.own = (8 * (r >> 2) + (r & 3)) * stride + 8 * c;
+    if constexpr (sizeof(T) == 2) {
+        t.k4 = (4 * c + (r >> 2)) * stride + 8 * (r & 3);
+        t.k8 = (8 * c + (r >> 2)) * stride + 8 * (r & 3);
+    } else {
+        t.k4 = 4 * c * stride + 8 * (r >> 2) + (r & 3);
+        t.k8 = 8 * c * stride + 8 * (r >> 2) + (r & 3);
+    }
+    return t;
+}
+// compile-time part of a transposed read: band starting at row `krow`, feature tile t
+__host__ __device__ constexpr int tr_const(int krow, int t, int stride)
+{
+    return krow * stride + 32 * (t >> 1) + 4 * (t & 1);
+}
+// compile-time part of a natural read of row pi(t, .) at feature offset f
+__host__ __device__ constexpr int own_const(int t, int f, int stride)
+{
+    return (32 * (t >> 1) + 4 * (t & 1)) * stride + f;
+}
+
+__device__ __forceinline__ bf16x4 lds_tr4(const __bf16 *p, int stride)
+{
+    (void)stride;
     typedef __attribute__((ext_vector_type(4))) short v4s;
     v4s v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)p);
     return __builtin_bit_cast(bf16x4, v);
 }
-__device__ __forceinline__ f32x4 lds_tr4(const float *tile, int stride, int krow0, int colseg, int colown)
+__device__ __forceinline__ f32x4 lds_tr4(const float *p, int stride)
 {
-    (void)colseg;
-    const float *p = tile + krow0 * stride + colown;
     f32x4 r = {p[0], p[stride], p[2 * stride], p[3 * stride]};
     return r;
 }
 
-// Column helpers for the feature permutation pi: tile t of a (feature x token) product.
-struct PiCols {
-    int seg, own;
-};
-__device__ __forceinline__ PiCols pi_cols(int t)
-{
-    const int r = threadIdx.x & 15;
-    PiCols p;
-    p.seg = 32 * (t >> 1) + 8 * (r & 3) + 4 * (t & 1);
-    p.own = 32 * (t >> 1) + 8 * (r >> 2) + 4 * (t & 1) + (r & 3);
-    return p;
-}
 // Plain mapping: tile t covers features 16t .. 16t+15, lane i gets feature 16t + i.
-__device__ __forceinline__ PiCols plain_cols(int t)
+template <typename T> __device__ __forceinline__ int plain_tr_lane(int stride)
 {
-    const int r = threadIdx.x & 15;
-    PiCols p;
-    p.seg = 16 * t + 4 * (r & 3);
-    p.own = 16 * t + r;
-    return p;
+    const int lane = threadIdx.x & 63, r = lane & 15, c = lane >> 4;
+    if constexpr (sizeof(T) == 2) return (4 * c + (r >> 2)) * stride + 4 * (r & 3);
+    else return 4 * c * stride + r;
 }
 
 // ---- gate prefix/suffix hierarchy inside a 16-token sub-block -------------------------------------

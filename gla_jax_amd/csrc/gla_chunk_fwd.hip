@@ -42,6 +42,8 @@ __global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restric
     const int N = T_len / C;
     const int64_t tok = (int64_t)b * T_len + (int64_t)n * C + 16 * w + r;
     const int64_t rowoff = (tok * H + h) * D;
+    const TrLane<T> L = make_tr_lane<T>(LS);
+    const int wrow = 16 * w * LS + L.nat;          // this lane's row of a [token][feature] tile
 
     float p[NV], s[NV];
     D8 qf[KS], kf[KS];
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restric
         for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
         qf[ks] = ld8(q + rowoff + d0);
         kf[ks] = ld8(k + rowoff + d0);
-        st8(Vn + (16 * w + r) * LS + d0, ld8(v + rowoff + d0));
+        st8(Vn + wrow + 32 * ks, ld8(v + rowoff + d0));
     }
     {
         const T *sp = states + (((int64_t)b * H + h) * N + n) * D * D;
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restric
                 qh[8 * ks + e] = a[e] * fast_exp2(p[8 * ks + e]);
                 kh[e] = bq[e] * fast_exp2(s[8 * ks + e]);
             }
-            st8(Kh + (16 * w + r) * LS + 32 * ks + 8 * c, pack8<T>(kh));
+            st8(Kh + wrow + 32 * ks, pack8<T>(kh));
         }
         dot = reduce_over_cgroups(dot);
 #pragma unroll
@@ -134,7 +136,7 @@ __global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restric
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 D8 qb = pack8<T>(qh + 8 * ks);
-                D8 ka = ld8(Kh + (16 * J + r) * LS + 32 * ks + 8 * c);
+                D8 ka = ld8(Kh + L.nat + 16 * J * LS + 32 * ks);
                 accT[J] = mma_d(ka, qb, accT[J]);
                 f32x8 rr = ld8(rtab + J * D + 32 * ks + 8 * c);
 #pragma unroll
@@ -153,7 +155,7 @@ __global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restric
         D8 qb = pack8<T>(qh + 8 * ks);   // q * exp(L_i)
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            D8 sa = ld8(St + pi_cols(t).own * LS + 32 * ks + 8 * c);
+            D8 sa = ld8(St + L.own + own_const(t, 32 * ks, LS));
             acc[t] = mma_d(sa, qb, acc[t]);
         }
     }
@@ -163,8 +165,7 @@ __global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restric
             auto b4 = pack4<T>(J == w ? accD : accT[J]);
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                const PiCols pc = pi_cols(t);
-                auto a4 = lds_tr4(Vn, LS, 16 * J + 4 * c, pc.seg, pc.own);
+                auto a4 = lds_tr4(Vn + L.k4 + tr_const(16 * J, t, LS), LS);
                 acc[t] = mma_t(a4, b4, acc[t]);
             }
         }

@@ -101,14 +101,13 @@ __global__ __launch_bounds__(C * 4) void chunk_outer_kernel(const float *__restr
         f32x4 acc[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const PiCols ca = plain_cols(mt);
+        const int ptl = plain_tr_lane<T>(LS);
 #pragma unroll 2
         for (int J = 0; J < NB; ++J) {
-            auto a = lds_tr4(Xn, LS, 16 * J + 4 * c, ca.seg, ca.own);
+            auto a = lds_tr4(Xn + ptl + 16 * J * LS + 16 * mt, LS);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const PiCols cb = plain_cols(nt);
-                auto bb = lds_tr4(Yn, LS, 16 * J + 4 * c, cb.seg, cb.own);
+                auto bb = lds_tr4(Yn + ptl + 16 * J * LS + 16 * nt, LS);
                 acc[nt] = mma_t(a, bb, acc[nt]);
             }
         }

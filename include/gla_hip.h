@@ -134,6 +134,24 @@ int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int
                   void *dhidden_init, float *dlog_fgate, void *dvalue, void *dkey, void *dquery,
                   void *workspace, size_t workspace_bytes);
 
+/* Same as gla_chunk_fwd / gla_chunk_bwd but launching only the kernels selected by `stages`
+ * (bit 0: per-chunk outer products, bit 1: scan over chunks, bit 2: output / gradient kernel), the
+ * others' results being taken from the workspace and residual buffers of an earlier full call with
+ * the same arguments.  No counterpart in the reference; exists so that a caller can time one kernel
+ * with events on its own stream (bench.py does). */
+int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                         int64_t chunk_size, gla_dtype dtype,
+                         const void *hidden_init, const float *log_fgate, const void *value,
+                         const void *key, const void *query,
+                         void *hidden_final, void *out, void *states,
+                         void *workspace, size_t workspace_bytes);
+int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                         int64_t chunk_size, gla_dtype dtype,
+                         const float *log_fgate, const void *value, const void *key, const void *query,
+                         const void *states, const void *dhidden_final, const void *dout,
+                         void *dhidden_init, float *dlog_fgate, void *dvalue, void *dkey, void *dquery,
+                         void *workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif
