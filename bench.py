@@ -223,6 +223,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="chunk", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run 3 plain device copies of 256 MiB (a kernel of known traffic, to scale "
+                         "rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures ONE GPU: every (batch, head) pair is an independent unit, a multi-GPU "
@@ -231,6 +234,13 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     kind, B, T, H, D, chunk, shift = WORKLOADS[args.workload]
+    if args.calibrate:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if kind == "chunk":
         r = bench_chunk(B, T, H, D, chunk, shift, args.steps, args.warmup)
         metric = "chunk_gla fwd+bwd Mtokens/s (B4,T4096,H6,D128 bf16); % bf16 MFMA peak" \

@@ -1,0 +1,97 @@
+"""CPU-side checks of the drop-in boundary: libgla_hip.so loads, exports every symbol that
+include/gla_hip.h declares, rejects bad arguments on the host before any launch, and the Python
+front-end refuses to run without the GPU path (there is no CPU fallback)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from gla_jax_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "gla_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gla_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_typed():
+    names = declared_symbols()
+    assert len(names) >= 13
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in gla_hip.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature in gla_jax_amd/_lib.py"
+    assert sorted(_lib.SIGNATURES) == names
+    assert _lib.load().gla_abi_version() == 1
+
+
+def test_status_strings():
+    for code in range(-7, 1):
+        assert len(_lib.status_string(code)) > 1
+    assert "chunk" in _lib.status_string(-4)
+
+
+def test_chunk_plan_and_sizes():
+    lib = _lib.load()
+    B, T, H, D = 4, 4096, 6, 128
+    n_chunks = T // 128
+    st = lib.gla_chunk_states_bytes(B, T, H, D, D, 128, _lib.GLA_BF16)
+    assert st == B * H * n_chunks * D * D * 2
+    ws = lib.gla_chunk_fwd_workspace_bytes(B, T, H, D, D, 128, _lib.GLA_BF16)
+    assert ws >= B * H * n_chunks * (D * D * 4 + D * 4) + st
+    # chunk sizes above the largest tile reuse it; unsupported combinations report 0
+    assert lib.gla_chunk_states_bytes(B, T, H, D, D, 256, _lib.GLA_BF16) == st
+    assert lib.gla_chunk_states_bytes(B, T, H, D, D, 96, _lib.GLA_BF16) == 0      # not a power of two
+    assert lib.gla_chunk_states_bytes(B, 100, H, D, D, 64, _lib.GLA_BF16) == 0    # does not divide T
+    assert lib.gla_chunk_states_bytes(B, T, H, 128, 64, 128, _lib.GLA_BF16) == 0  # DK != DV
+    assert lib.gla_chunk_states_bytes(B, T, H, D, D, 128, _lib.GLA_F32) == 0      # fp32 is built for D=64
+
+
+def test_entry_points_reject_bad_arguments_without_touching_the_gpu():
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    a = (ctypes.addressof(buf) + 15) & ~15          # a 16-byte aligned, non-null host address (never dereferenced)
+    # NULL pointers
+    assert lib.gla_cumsum_f32(None, None, None, a, 1, 8, 8, 0) == -1
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 1, 1, 0, None, a, a, a, a, a, a) == -1
+    # shapes / dtypes
+    assert lib.gla_cumsum_f32(None, a, None, a, 0, 8, 8, 0) == -2
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 48, 48, 1, 1, 0, a, a, a, a, a, a, a) == -2
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 32, 1, 1, 0, a, a, a, a, a, a, a) == -2   # DK != DV
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 5, 1, 0, a, a, a, a, a, a, a) == -3
+    assert lib.gla_rnn_scan_f32(None, a, a, None, None, None, a, 1, 4, 4, 3, 0) == -2          # V % 4
+    # misaligned
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 1, 1, 0, a + 2, a, a, a, a, a, a) == -6
+    # chunk: not a power of two / not dividing T / unsupported head dim / missing workspace
+    args = lambda T, D, C: (None, 1, T, 1, D, D, C, 1, a, a, a, a, a, a, a, a)
+    assert lib.gla_chunk_fwd(*args(256, 64, 48), a, 1 << 30) == -4
+    assert lib.gla_chunk_fwd(*args(200, 64, 64), a, 1 << 30) == -4
+    assert lib.gla_chunk_fwd(*args(256, 96, 64), a, 1 << 30) == -7
+    assert lib.gla_chunk_fwd(*args(256, 64, 64), None, 0) == -5
+    assert lib.gla_chunk_fwd(*args(256, 64, 64), a, 16) == -5
+    assert lib.gla_chunk_bwd(None, 1, 256, 1, 64, 64, 64, 1, a, a, a, a, None, a, a, a, a, a, a, a, a, 1 << 30) == -1
+
+
+def test_front_end_has_no_cpu_path():
+    from gla_jax_amd import chunk_gla, cumsum_recursive, recurrent_gla
+    T, H, D = 64, 1, 64
+    h0 = torch.zeros(H, D, D)
+    x = torch.zeros(T, H, D)
+    with pytest.raises(ValueError, match="GPU"):
+        chunk_gla(h0, x, x, x, x, 64)
+    with pytest.raises(ValueError, match="GPU"):
+        recurrent_gla(h0, x, x, x, x)
+    with pytest.raises(ValueError, match="GPU"):
+        cumsum_recursive(x, 0)
+
+
+def test_oracle_is_not_imported_by_the_product():
+    import glob
+    for f in glob.glob(os.path.join(ROOT, "gla_jax_amd", "*.py")):
+        src = open(f).read()
+        assert "oracle" not in src, f"{f} mentions the oracle: the product path must not depend on it"
