@@ -42,25 +42,6 @@ __device__ __forceinline__ f32x8 join4(f32x4 lo, f32x4 hi)
     return r;
 }
 
-// Hides a pointer's provenance from the optimiser: loads through the result are not merged with
-// earlier loads of (or forwarded from earlier stores to) the same address, so a value can be dropped
-// from registers and fetched again (an L2 hit) where it is needed next.
-template <typename P> __device__ __forceinline__ P *refetch(P *ptr)
-{
-    asm volatile("" : "+v"(ptr));
-    return ptr;
-}
-
-// inclusive suffix sum over the 16 token rows of the wave (lane r receives sum over rows >= r)
-__device__ __forceinline__ float suffix_sum_rows(float x)
-{
-    x += dpp_f32<0x101>(x);   // row_shl:1, lanes past the row end read 0
-    x += dpp_f32<0x102>(x);
-    x += dpp_f32<0x104>(x);
-    x += dpp_f32<0x108>(x);
-    return x;
-}
-
 template <typename T, int C, int D>
 __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k,
@@ -83,6 +64,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     float *rtab = reinterpret_cast<float *>(xs + NB * 16 * XS);   // [NB][D] e^{tau_m}
     float *dltab = rtab + NB * D;                  // [NB][D] sub-block sums of the gate-cumsum gradient
     float *lbar = dltab + NB * D;                  // [D] chunk-level gate gradient
+    float *ttab = lbar + D;                        // [NB][D] tau_m (log2 units)
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: scalar branches on it
@@ -100,6 +82,8 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     D8 dof[KS];
     f32x4 Aown = {0.f, 0.f, 0.f, 0.f};   // scores A[i = 4c+e][j = r] of the own sub-block
     T4 symb[4];                          // per level: masked (dA + dA^T) of the own sub-block, MFMA operand
+                                         // (one anchor: [0] = dA^T below the diagonal, [1] = dA below it)
+    bool one_anchor;                     // wave-uniform: the sub-block's gates are mild enough for ONE anchor
     float dd = 0.f;                      // dA_ii of this lane's row
     {
         float p[NV], s[NV];
@@ -109,7 +93,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             const int d0 = 32 * ks + 8 * c;
             f32x8 gg = ld8(g + rowoff + d0);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
+            for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
             qf[ks] = ld8(q + rowoff + d0);
             kf[ks] = ld8(k + rowoff + d0);
             vf[ks] = ld8(v + rowoff + d0);
@@ -138,8 +122,31 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
 #pragma unroll
         for (int e = 0; e < 4; ++e) Aown[e] = (4 * c + e == r) ? dot : 0.f;   // A_ii = q_i.k_i (gla.py:983)
 
-        // Pass 1 over the dyadic levels, full head dimension: the mixed tile X of every level -> the
-        // level's score blocks (they contract over all features), and the gate prefix/suffix sums.
+        // p = l_i (inclusive prefix over the 16 rows, log2 units), s = tau - l_i; the totals go through
+        // the wave's row of ttab (same-wave LDS accesses execute in order) and stay there.
+#pragma unroll
+        for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
+        if (r == 15) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) st8(ttab + w * D + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
+        }
+        asm volatile("" ::: "memory");
+        {
+            float span = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                f32x8 tau = ld8(ttab + w * D + 32 * ks + 8 * c);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    s[8 * ks + e] = tau.v[e] - p[8 * ks + e];
+                    span = fmaxf(span, fmaxf(fabsf(p[8 * ks + e]), fabsf(s[8 * ks + e])));
+                }
+            }
+            one_anchor = wave_all_below(span, kOneAnchorSpan);
+        }
+
+        // Harder gates: pass 1 over the dyadic levels, full head dimension: the mixed tile X of every level
+        // -> the level's score blocks (they contract over all features), and the gate prefix/suffix sums.
         auto level_scores = [&](auto hc, auto lc) {
             constexpr int h_ = decltype(hc)::value, L_ = decltype(lc)::value;
             const bool upper = (r & h_) != 0;
@@ -168,10 +175,18 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             hier_step<h_>(p, s, upper);
             __builtin_amdgcn_sched_barrier(0);
         };
-        level_scores(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
-        level_scores(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
-        level_scores(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
-        level_scores(std::integral_constant<int, 8>{}, std::integral_constant<int, 3>{});
+        if (!one_anchor) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                f32x8 gg = ld8(refetch(g + rowoff) + 32 * ks + 8 * c);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
+            }
+            level_scores(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+            level_scores(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
+            level_scores(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
+            level_scores(std::integral_constant<int, 8>{}, std::integral_constant<int, 3>{});
+        }
 
         // p = l_i, s = tau - l_i (log2 units): table of e^{tau}, rescaled key and query tiles
         if (r == 0) {
@@ -183,18 +198,35 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 st8(rtab + w * D + 32 * ks + 8 * c, t);
             }
         }
+        // One anchor (the end of the sub-block): A_ij = [q_i e^{l_i - tau}] . [k_j e^{tau - l_j}]; the key
+        // factor is the operand of the other sub-blocks as well.
+        f32x4 G = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            float a[8], bq[8];
+            float a[8], bq[8], qo[8];
             unpack8(qf[ks], a);
             unpack8(kf[ks], bq);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
+                qo[e] = a[e] * fast_exp2(-s[8 * ks + e]);
                 a[e] *= fast_exp2(p[8 * ks + e]);
                 bq[e] *= fast_exp2(s[8 * ks + e]);
             }
+            const D8 kh = pack8<T>(bq);
             st8(tile3 + wrow + 32 * ks, pack8<T>(a));
-            st8(tile1 + wrow + 32 * ks, pack8<T>(bq));
+            st8(tile1 + wrow + 32 * ks, kh);
+            if (one_anchor) G = mma_d(pack8<T>(qo), kh, G);
+        }
+        if (one_anchor) {
+            f32x4 lowT, low;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                Aown[e] += (4 * c + e > r) ? G[e] : 0.f;
+                lowT[e] = (4 * c + e < r) ? dAt[e] : 0.f;
+                low[e] = (4 * c + e > r) ? dAn[e] : 0.f;
+            }
+            symb[0] = pack4<T>(lowT);
+            symb[1] = pack4<T>(low);
         }
         const T *sp = states + bhn * D * D;
         for (int idx = threadIdx.x; idx < D * D / 8; idx += C * 4) {
@@ -278,10 +310,43 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             asm volatile("" ::: "memory");
             hier_step<h_>(p8, s8, upper);
         };
-        slice_level(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
-        slice_level(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
-        slice_level(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
-        slice_level(std::integral_constant<int, 8>{}, std::integral_constant<int, 3>{});
+        if (one_anchor) {
+            // the own sub-block is one more link on either side: dq~ = dA k~, dk~ = dA^T q~ (below the diagonal)
+            f32x8 tau = ld8(ttab + w * D + fo + 8 * c);
+            float fq[8], fk[8], x[8], xr[8], kr[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                p8[e] = prefix_sum_rows(p8[e]);
+                s8[e] = tau.v[e] - p8[e];
+                fq[e] = fast_exp2(-s8[e]);
+                fk[e] = fast_exp2(s8[e]);
+                x[e] = a[e] * fq[e];
+                kr[e] = bq[e] * fk[e];
+            }
+            D8 X = pack8<T>(x);
+            unpack8(X, xr);
+            unpack8(pack8<T>(kr), kr);
+            st8(xw + Lx.nat, X);
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                f32x4 z4 = {0.f, 0.f, 0.f, 0.f};
+                f32x4 gq = mma_t(lds_tr4(tile1 + L.k4 + fo + 4 * tt + 16 * w * LS, LS), symb[0], z4);
+                f32x4 hk = mma_t(lds_tr4(xw + Lx.k4 + 4 * tt, XS), symb[1], z4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    dq8[4 * tt + e] += gq[e] * fq[4 * tt + e];
+                    dk8[4 * tt + e] += hk[e] * fk[4 * tt + e];
+                    dl8[4 * tt + e] += gq[e] * xr[4 * tt + e] - hk[e] * kr[4 * tt + e];
+                }
+            }
+            asm volatile("" ::: "memory");
+        } else {
+            slice_level(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+            slice_level(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
+            slice_level(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
+            slice_level(std::integral_constant<int, 8>{}, std::integral_constant<int, 3>{});
+        }
         {
             f32x8 pk;
 #pragma unroll
@@ -474,17 +539,14 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                     }
                 }
             }
-            // epilogue: e^{tau - l} of the slice is rebuilt from the gates (4 prefix/suffix steps)
-            float p8[8], s8[8], o[8];
+            // epilogue: e^{tau - l} of the slice is rebuilt from the gates
+            float s8[8], o[8];
             {
                 f32x8 gg = ld8(refetch(g + rowoff) + fo + 8 * c);
+                f32x8 tau = ld8(ttab + w * D + fo + 8 * c);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) { p8[e] = gg.v[e] * kLog2e; s8[e] = 0.f; }
+                for (int e = 0; e < 8; ++e) s8[e] = tau.v[e] - prefix_sum_rows(gg.v[e] * kLog2e);
             }
-            hier_step<1>(p8, s8, (r & 1) != 0);
-            hier_step<2>(p8, s8, (r & 2) != 0);
-            hier_step<4>(p8, s8, (r & 4) != 0);
-            hier_step<8>(p8, s8, (r & 8) != 0);
             f32x8 parked = ld8(refetch(dg + rowoff) + fo + 8 * c);
             f32x8 sfx;
 #pragma unroll
@@ -527,7 +589,7 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
     constexpr int XS = 32 + 16 / (int)sizeof(T);
     constexpr int TR = C > D ? C : D, NB = C / 16;
     const size_t lds = ((size_t)4 * TR * LS + (size_t)NB * 16 * XS) * sizeof(T) +
-                       (size_t)(2 * NB + 1) * D * sizeof(float);
+                       (size_t)(3 * NB + 1) * D * sizeof(float);
     auto kern = chunk_grad_kernel<T, C, D>;
     if (int e = allow_lds((const void *)kern, lds)) return e;
     dim3 grid(T_len / C, H, B), block(C * 4);

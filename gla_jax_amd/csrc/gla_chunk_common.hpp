@@ -203,6 +203,47 @@ template <int H, int NV> __device__ __forceinline__ void hier_step(float (&p)[NV
     }
 }
 
+// Inclusive prefix / suffix sum over the 16 token rows of the wave (lanes of one DPP row): lane r
+// receives the sum over rows <= r (>= r).  Lanes shifted in from outside the row read 0.
+__device__ __forceinline__ float prefix_sum_rows(float x)
+{
+    x += dpp_f32<0x111>(x);   // row_shr:1
+    x += dpp_f32<0x112>(x);
+    x += dpp_f32<0x114>(x);
+    x += dpp_f32<0x118>(x);
+    return x;
+}
+__device__ __forceinline__ float suffix_sum_rows(float x)
+{
+    x += dpp_f32<0x101>(x);   // row_shl:1
+    x += dpp_f32<0x102>(x);
+    x += dpp_f32<0x104>(x);
+    x += dpp_f32<0x108>(x);
+    return x;
+}
+
+// A sub-block whose gate sums stay below this many powers of two (in either direction, for every
+// feature and every row) is handled with ONE anchor instead of the dyadic recursion: its rescaled
+// operands are at most 2^48 and their products cannot overflow.  log_sigmoid gates reach this only
+// when they average below -2 nats per token over 16 tokens; harder gates (up to outright resets) take
+// the recursion, whose factors never exceed 1.
+constexpr float kOneAnchorSpan = 48.f;
+
+// Wave-uniform: true if x < limit on every lane (a NaN counts as not below).
+__device__ __forceinline__ bool wave_all_below(float x, float limit)
+{
+    return __ballot(!(x < limit)) == 0ull;
+}
+
+// Hides a pointer's provenance from the optimiser: loads through the result are not merged with
+// earlier loads of (or forwarded from earlier stores to) the same address, so a value can be dropped
+// from registers and fetched again (an L2 hit) where it is needed next.
+template <typename P> __device__ __forceinline__ P *refetch(P *ptr)
+{
+    asm volatile("" : "+v"(ptr));
+    return ptr;
+}
+
 // Sum over the 4 lanes (c = 0..3) that hold the same token row.
 __device__ __forceinline__ float reduce_over_cgroups(float x)
 {

@@ -52,7 +52,7 @@ __global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restric
         const int d0 = 32 * ks + 8 * c;
         f32x8 gg = ld8(g + rowoff + d0);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
+        for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
         qf[ks] = ld8(q + rowoff + d0);
         kf[ks] = ld8(k + rowoff + d0);
         st8(Vn + wrow + 32 * ks, ld8(v + rowoff + d0));
@@ -65,35 +65,86 @@ __global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restric
         }
     }
 
-    // ---- inside the sub-block: dyadic levels 2, 4, 8, 16 -----------------------------------------
+    // ---- gate prefix of the sub-block; can the whole sub-block share ONE anchor? ------------------
+    // p = l_i (inclusive prefix over the 16 rows, log2 units), s = tau - l_i.  The totals travel through
+    // the wave's own row of rtab (same-wave LDS accesses execute in order).
+#pragma unroll
+    for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
+    if (r == 15) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) st8(rtab + w * D + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
+    }
+    asm volatile("" ::: "memory");
+    float span = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        f32x8 tau = ld8(rtab + w * D + 32 * ks + 8 * c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            s[8 * ks + e] = tau.v[e] - p[8 * ks + e];
+            span = fmaxf(span, fmaxf(fabsf(p[8 * ks + e]), fabsf(s[8 * ks + e])));
+        }
+    }
+    asm volatile("" ::: "memory");
+    const bool one_anchor = wave_all_below(span, kOneAnchorSpan);
+
     f32x4 accD = {0.f, 0.f, 0.f, 0.f};   // transposed scores of the diagonal sub-block: [j = 4c+e][i = r]
-    auto level = [&](auto hc) {
-        constexpr int h_ = decltype(hc)::value;
-        const bool upper = (r & h_) != 0;
+    if (one_anchor) {
+        // Gates this mild need no recursion: with the anchor at the end of the sub-block,
+        // A_ij = [q_i e^{l_i - tau}] . [k_j e^{tau - l_j}], both factors are finite (at most 2^span) and carry
+        // the same relative rounding as the dyadic form.  The key factor is the operand of the other
+        // sub-blocks as well.
         f32x4 G = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            float a[8], bq[8], x[8];
+            float a[8], bq[8];
             unpack8(qf[ks], a);
             unpack8(kf[ks], bq);
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-                x[e] = upper ? a[e] * fast_exp2(p[8 * ks + e]) : bq[e] * fast_exp2(s[8 * ks + e]);
-            D8 X = pack8<T>(x);
-            G = mma_d(X, X, G);
+            for (int e = 0; e < 8; ++e) {
+                a[e] *= fast_exp2(-s[8 * ks + e]);
+                bq[e] *= fast_exp2(s[8 * ks + e]);
+            }
+            G = mma_d(pack8<T>(bq), pack8<T>(a), G);
         }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int j = 4 * c + e;
-            const bool ok = ((j ^ r) < 2 * h_) && upper && !(j & h_);
-            accD[e] += ok ? G[e] : 0.f;
+        for (int e = 0; e < 4; ++e) accD[e] = (4 * c + e < r) ? G[e] : 0.f;
+    } else {
+        // ---- the dyadic levels 2, 4, 8, 16 of the reference ------------------------------------------
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            f32x8 gg = ld8(refetch(g + rowoff) + 32 * ks + 8 * c);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
         }
-        hier_step<h_>(p, s, upper);
-    };
-    level(std::integral_constant<int, 1>{});
-    level(std::integral_constant<int, 2>{});
-    level(std::integral_constant<int, 4>{});
-    level(std::integral_constant<int, 8>{});
+        auto level = [&](auto hc) {
+            constexpr int h_ = decltype(hc)::value;
+            const bool upper = (r & h_) != 0;
+            f32x4 G = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                float a[8], bq[8], x[8];
+                unpack8(qf[ks], a);
+                unpack8(kf[ks], bq);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    x[e] = (upper ? a[e] : bq[e]) * fast_exp2(upper ? p[8 * ks + e] : s[8 * ks + e]);
+                D8 X = pack8<T>(x);
+                G = mma_d(X, X, G);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int j = 4 * c + e;
+                const bool ok = ((j ^ r) < 2 * h_) && upper && !(j & h_);
+                accD[e] += ok ? G[e] : 0.f;
+            }
+            hier_step<h_>(p, s, upper);
+        };
+        level(std::integral_constant<int, 1>{});
+        level(std::integral_constant<int, 2>{});
+        level(std::integral_constant<int, 4>{});
+        level(std::integral_constant<int, 8>{});
+    }
 
     // p = l_i (inclusive, log2 units), s = tau - l_i.  Rescaled operands, diagonal, table of exp(tau).
     float qh[NV];
