@@ -53,6 +53,8 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     constexpr int LS = TileGeom<T, D>::kStride;
     constexpr int XS = 32 + 16 / (int)sizeof(T);   // row stride of the per-wave slice scratch
     constexpr int TR = C > D ? C : D;              // rows of one LDS tile
+    constexpr int SR = (D * D / 8) / (C * 4);      // 16-byte pieces of a D x D state per thread
+    static_assert(SR * C * 4 * 8 == D * D, "state staging assumes whole pieces per thread");
     typedef typename FragTypes<T>::d8 D8;
     typedef typename FragTypes<T>::t4 T4;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -69,7 +71,9 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: scalar branches on it
     const int r = lane & 15, c = lane >> 4;
-    const int n = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    // heads vary fastest over the grid: workgroups that run together touch the same DRAM pages of the
+    // [B, T, H, D] arrays (a token's H rows are contiguous)
+    const int h = blockIdx.x % H, n = blockIdx.x / H, b = blockIdx.y;
     const int N = T_len / C;
     const int64_t tok = (int64_t)b * T_len + (int64_t)n * C + 16 * w + r;
     const int64_t rowoff = (tok * H + h) * D;
@@ -78,6 +82,10 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const TrLane<T> Lx = make_tr_lane<T>(XS);
     const int wrow = 16 * w * LS + L.nat;          // this lane's row of a [token][feature] tile
     T *xw = xs + w * 16 * XS;                      // [16][XS]: one 32-feature slice of the wave's rows
+
+    // Piece i of a D x D state that this thread moves between global memory and its LDS tile.
+    const int st_row = threadIdx.x / (D / 8), st_c8 = (threadIdx.x % (D / 8)) * 8;
+    constexpr int kStRows = C * 4 / (D / 8);       // rows covered by one round of the workgroup
 
     D8 dof[KS];
     f32x4 Aown = {0.f, 0.f, 0.f, 0.f};   // scores A[i = 4c+e][j = r] of the own sub-block
@@ -99,6 +107,13 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             vf[ks] = ld8(v + rowoff + d0);
             dof[ks] = ld8(dout + rowoff + d0);
             st8(tile0 + wrow + 32 * ks, vf[ks]);
+        }
+        // the chunk-start state is requested now and lands in its tile just before the first barrier
+        D8 sreg[SR];
+        {
+            const T *sp = states + bhn * D * D;
+#pragma unroll
+            for (int i = 0; i < SR; ++i) sreg[i] = ld8(sp + (st_row + i * kStRows) * D + st_c8);
         }
         if (threadIdx.x < D) lbar[threadIdx.x] = 0.f;
 
@@ -228,15 +243,15 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             symb[0] = pack4<T>(lowT);
             symb[1] = pack4<T>(low);
         }
-        const T *sp = states + bhn * D * D;
-        for (int idx = threadIdx.x; idx < D * D / 8; idx += C * 4) {
-            const int row = idx / (D / 8), c8 = (idx % (D / 8)) * 8;
-            st8(tile2 + row * LS + c8, ld8(sp + row * D + c8));
-        }
+#pragma unroll
+        for (int i = 0; i < SR; ++i) st8(tile2 + (st_row + i * kStRows) * LS + st_c8, sreg[i]);
     }
     __syncthreads();
 
     // ---- row-owner role ----------------------------------------------------------------------------
+    // Per-row inputs of a slice are fetched one slice ahead (L2 hits, but still a microsecond away).
+    f32x8 gN = ld8(refetch(g + rowoff) + 8 * c);
+    D8 qN = ld8(refetch(q + rowoff) + 8 * c), kN = ld8(refetch(k + rowoff) + 8 * c);
     // score blocks dA^T of the earlier sub-blocks: dAT_J[j][i] = v_j . dO_i  (J < w)
     T4 dATc[NB];
 #pragma unroll
@@ -265,11 +280,15 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
         const int fo = 32 * ks;
         float p8[8], s8[8], a[8], bq[8], dq8[8], dk8[8], dl8[8];
         {
-            f32x8 gg = ld8(refetch(g + rowoff) + fo + 8 * c);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { p8[e] = gg.v[e] * kLog2e; s8[e] = 0.f; }
-            unpack8(ld8(refetch(q + rowoff) + fo + 8 * c), a);
-            unpack8(ld8(refetch(k + rowoff) + fo + 8 * c), bq);
+            for (int e = 0; e < 8; ++e) { p8[e] = gN.v[e] * kLog2e; s8[e] = 0.f; }
+            unpack8(qN, a);
+            unpack8(kN, bq);
+            if (ks + 1 < KS) {
+                gN = ld8(refetch(g + rowoff) + fo + 32 + 8 * c);
+                qN = ld8(refetch(q + rowoff) + fo + 32 + 8 * c);
+                kN = ld8(refetch(k + rowoff) + fo + 32 + 8 * c);
+            }
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -400,30 +419,47 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             }
         }
     }
+    // What the column-owner loop needs per slice (the parked values and the gates), again one slice ahead.
+    f32x8 gN2, dlN, pkN;
+    auto fetch_parked = [&](int fo) {
+        gN2 = ld8(refetch(g + rowoff) + fo + 8 * c);
+        pkN = ld8(refetch(dg + rowoff) + fo + 8 * c);
+        if constexpr (sizeof(T) == 2) {
+            dlN = join4(*reinterpret_cast<const f32x4 *>(refetch(dk + rowoff) + fo + 8 * c),
+                        *reinterpret_cast<const f32x4 *>(refetch(dv + rowoff) + fo + 8 * c));
+        } else {
+            dlN = ld8(reinterpret_cast<const float *>(refetch(dk + rowoff) + fo + 8 * c));
+        }
+    };
+    fetch_parked(0);
+    D8 dsreg[SR];                                  // dS' of the chunk, requested before the barrier
+    {
+        const T *dsp = dstates + bhn * D * D;
+#pragma unroll
+        for (int i = 0; i < SR; ++i) dsreg[i] = ld8(dsp + (st_row + i * kStRows) * D + st_c8);
+    }
+    const f32x8 dec = ld8(decay + bhn * D + st_c8);
     __syncthreads();
 
     // ---- second set of tiles: dO, dS'^T; chunk-level term sum_v S*dS' ------------------------------
     {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) st8(tile0 + wrow + 32 * ks, dof[ks]);
-        const T *dsp = dstates + bhn * D * D;
         float part[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) part[e] = 0.f;
-        const int c8 = (threadIdx.x % (D / 8)) * 8;
-        for (int idx = threadIdx.x; idx < D * D / 8; idx += C * 4) {
-            const int row = idx / (D / 8);
-            D8 dsv = ld8(dsp + row * D + c8);
+#pragma unroll
+        for (int i = 0; i < SR; ++i) {
+            T *cell = tile2 + (st_row + i * kStRows) * LS + st_c8;
             float a[8], bq[8];
-            unpack8(ld8(tile2 + row * LS + c8), a);
-            unpack8(dsv, bq);
+            unpack8(ld8(cell), a);
+            unpack8(dsreg[i], bq);
 #pragma unroll
             for (int e = 0; e < 8; ++e) part[e] += a[e] * bq[e];
-            st8(tile2 + row * LS + c8, dsv);
+            st8(cell, dsreg[i]);
         }
-        f32x8 dec = ld8(decay + bhn * D + c8);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) atomicAdd(lbar + c8 + e, part[e] * dec.v[e]);
+        for (int e = 0; e < 8; ++e) atomicAdd(lbar + st_c8 + e, part[e] * dec.v[e]);
     }
     __syncthreads();
 
@@ -467,13 +503,8 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     for (int ks = 0; ks < KS; ++ks) {
         const int fo = 32 * ks;
         // what the row-owner loop parked for this slice (read before the rows are overwritten below)
-        f32x8 dlq;
-        if constexpr (sizeof(T) == 2) {
-            dlq = join4(*reinterpret_cast<const f32x4 *>(refetch(dk + rowoff) + fo + 8 * c),
-                        *reinterpret_cast<const f32x4 *>(refetch(dv + rowoff) + fo + 8 * c));
-        } else {
-            dlq = ld8(reinterpret_cast<const float *>(refetch(dk + rowoff) + fo + 8 * c));
-        }
+        const f32x8 dlq = dlN, parked = pkN, gg = gN2;
+        if (ks + 1 < KS) fetch_parked(fo + 32);
         // dv slice
         {
             f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
@@ -542,12 +573,10 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             // epilogue: e^{tau - l} of the slice is rebuilt from the gates
             float s8[8], o[8];
             {
-                f32x8 gg = ld8(refetch(g + rowoff) + fo + 8 * c);
                 f32x8 tau = ld8(ttab + w * D + fo + 8 * c);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) s8[e] = tau.v[e] - prefix_sum_rows(gg.v[e] * kLog2e);
             }
-            f32x8 parked = ld8(refetch(dg + rowoff) + fo + 8 * c);
             f32x8 sfx;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -561,6 +590,12 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             if (r == 0) st8(dltab + w * D + fo + 8 * c, sfx);
         }
     }
+    f32x8 own[KS];                                 // the row's suffix sums, parked by the loop above
+    {
+        const float *dgp = refetch(dg + rowoff);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) own[ks] = ld8(dgp + 32 * ks + 8 * c);
+    }
     __syncthreads();
 
     // ---- dlog_fgate = reverse cumsum over the whole chunk + the chunk-level term (gla.py:782) ------------
@@ -568,9 +603,8 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     for (int ks = 0; ks < KS; ++ks) {
         const int d0 = 32 * ks + 8 * c;
         f32x8 o = ld8(lbar + d0);
-        f32x8 own = ld8(refetch(dg + rowoff) + d0);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o.v[e] += own.v[e];
+        for (int e = 0; e < 8; ++e) o.v[e] += own[ks].v[e];
         for (int m = w + 1; m < NB; ++m) {
             f32x8 t = ld8(dltab + m * D + d0);
 #pragma unroll
@@ -592,7 +626,7 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
                        (size_t)(3 * NB + 1) * D * sizeof(float);
     auto kern = chunk_grad_kernel<T, C, D>;
     if (int e = allow_lds((const void *)kern, lds)) return e;
-    dim3 grid(T_len / C, H, B), block(C * 4);
+    dim3 grid(T_len / C * H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
                        (const T *)dout, (const T *)states, (const T *)dstates, decay, dg, (T *)dv, (T *)dk,
                        (T *)dq, T_len, H);

@@ -38,7 +38,9 @@ __global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restric
 
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int r = lane & 15, c = lane >> 4;
-    const int n = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    // heads vary fastest over the grid: workgroups that run together touch the same DRAM pages of the
+    // [B, T, H, D] arrays (a token's H rows are contiguous)
+    const int h = blockIdx.x % H, n = blockIdx.x / H, b = blockIdx.y;
     const int N = T_len / C;
     const int64_t tok = (int64_t)b * T_len + (int64_t)n * C + 16 * w + r;
     const int64_t rowoff = (tok * H + h) * D;
@@ -238,7 +240,7 @@ int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, co
     const size_t lds = (size_t)(2 * C + D) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
     auto kern = chunk_out_kernel<T, C, D>;
     if (int e = allow_lds((const void *)kern, lds)) return e;
-    dim3 grid(T_len / C, H, B), block(C * 4);
+    dim3 grid(T_len / C * H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
                        (const T *)states, (T *)out, T_len, H);
     return launch_status();

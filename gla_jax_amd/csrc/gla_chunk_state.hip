@@ -33,7 +33,9 @@ __global__ __launch_bounds__(C * 4) void chunk_outer_kernel(const float *__restr
 
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int r = lane & 15, c = lane >> 4;
-    const int n = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    // heads vary fastest over the grid: workgroups that run together touch the same DRAM pages of the
+    // [B, T, H, D] arrays (a token's H rows are contiguous)
+    const int h = blockIdx.x % H, n = blockIdx.x / H, b = blockIdx.y;
     const int N = T_len / C;
     const int64_t tok = (int64_t)b * T_len + (int64_t)n * C + 16 * w + r;
     const int64_t rowoff = (tok * H + h) * D;
@@ -171,7 +173,7 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
 {
     constexpr int LS = TileGeom<T, D>::kStride;
     const size_t lds = (size_t)2 * C * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
-    dim3 grid(T_len / C, H, B), block(C * 4);
+    dim3 grid(T_len / C * H, B), block(C * 4);
     if (mode == 0) {
         auto kern = chunk_outer_kernel<T, C, D, 0>;
         if (int e = allow_lds((const void *)kern, lds)) return e;
