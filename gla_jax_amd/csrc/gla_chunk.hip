@@ -67,7 +67,7 @@ extern "C" size_t gla_chunk_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H,
                                                 int64_t chunk_size, gla_dtype dtype)
 {
     ChunkPlan p;
-    // room for the chunk states as well, used when the caller keeps no residual
+    // per-chunk products, decays, and the chunk-start states in [dv][dk] orientation for the output kernel
     return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.prod + p.decay + p.states : 0;
 }
 
@@ -75,7 +75,8 @@ extern "C" size_t gla_chunk_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H,
                                                 int64_t chunk_size, gla_dtype dtype)
 {
     ChunkPlan p;
-    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.prod + p.decay + p.states : 0;
+    // per-chunk products, decays, and d(chunk-end state) in both orientations
+    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.prod + p.decay + 2 * p.states : 0;
 }
 
 extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK,
@@ -92,12 +93,12 @@ extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t
         if (!ptr) return GLA_ERR_NULL;
         if (!aligned16(ptr)) return GLA_ERR_ALIGN;
     }
-    if (!workspace || workspace_bytes < p.prod + p.decay + (states ? 0 : p.states)) return GLA_ERR_WORKSPACE;
+    if (!workspace || workspace_bytes < p.prod + p.decay + p.states) return GLA_ERR_WORKSPACE;
     if (!aligned16(workspace) || (states && !aligned16(states))) return GLA_ERR_ALIGN;
     unsigned char *ws = (unsigned char *)workspace;
     float *prodT = (float *)ws;
     float *decay = (float *)(ws + p.prod);
-    void *st_buf = states ? states : (void *)(ws + p.prod + p.decay);
+    void *statesT = (void *)(ws + p.prod + p.decay);   // [dv][dk], consumed by the output kernel
     hipStream_t st = (hipStream_t)stream;
     const int N = (int)(T / p.C);
     return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d) -> int {
@@ -108,10 +109,11 @@ extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t
             e = launch_chunk_outer<E, C_, D_>(st, 0, (int)B, (int)T, (int)H, log_fgate, value, key, prodT, decay);
         if (e) return e;
         if (stages & 2)
-            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 0, hidden_init, prodT, decay, st_buf, hidden_final);
+            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 0, hidden_init, prodT, decay, statesT, states,
+                                         hidden_final);
         if (e) return e;
         if (stages & 4)
-            e = launch_chunk_out<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, st_buf, out);
+            e = launch_chunk_out<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, statesT, out);
         return e;
     });
 }
@@ -142,12 +144,13 @@ extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t
         if (!ptr) return GLA_ERR_NULL;
         if (!aligned16(ptr)) return GLA_ERR_ALIGN;
     }
-    if (!workspace || workspace_bytes < p.prod + p.decay + p.states) return GLA_ERR_WORKSPACE;
+    if (!workspace || workspace_bytes < p.prod + p.decay + 2 * p.states) return GLA_ERR_WORKSPACE;
     if (!aligned16(workspace)) return GLA_ERR_ALIGN;
     unsigned char *ws = (unsigned char *)workspace;
     float *prodT = (float *)ws;
     float *decay = (float *)(ws + p.prod);
-    void *dstates = (void *)(ws + p.prod + p.decay);
+    void *dstatesT = (void *)(ws + p.prod + p.decay);            // d(chunk-end state), [dv][dk]
+    void *dstatesN = (void *)(ws + p.prod + p.decay + p.states); // the same, [dk][dv]
     hipStream_t st = (hipStream_t)stream;
     const int N = (int)(T / p.C);
     return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d) -> int {
@@ -158,11 +161,12 @@ extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t
             e = launch_chunk_outer<E, C_, D_>(st, 1, (int)B, (int)T, (int)H, log_fgate, dout, query, prodT, decay);
         if (e) return e;
         if (stages & 2)
-            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 1, dhidden_final, prodT, decay, dstates, dhidden_init);
+            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 1, dhidden_final, prodT, decay, dstatesT, dstatesN,
+                                         dhidden_init);
         if (e) return e;
         if (stages & 4)
             e = launch_chunk_grad<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,
-                                             states, dstates, decay, dlog_fgate, dvalue, dkey, dquery);
+                                             states, dstatesT, dstatesN, decay, dlog_fgate, dvalue, dkey, dquery);
         return e;
     });
 }

@@ -6,12 +6,13 @@
 //     and the chunk decay exp(L_end) per feature.
 //   chunk_scan_kernel    over chunks:  S_{n+1} = decay_n * S_n + P_n  (ops.py:286-297 combine op), written
 //     as the chunk-START states the output kernel needs (gla.py:720-723); run backwards it is the
-//     reverse scan of gla.py:759-765 and yields the gradient w.r.t. every chunk-END state.
+//     reverse scan of gla.py:759-765 and yields the gradient w.r.t. every chunk-END state.  Both
+//     orientations of the state are written, each consumer reads the one whose rows it contracts.
 //
 // L is the within-chunk inclusive cumsum of log_fgate (gla.py:509), never written to memory: each
 // wave scans its 16 tokens across lanes, block totals go through a small LDS table.
-// States are kept transposed, [dv][dk], because they are consumed as the A operand of
-// (feature x token) products contracting over dk.
+// States are consumed as the A operand of (feature x token) products: [dv][dk] where the product
+// contracts over dk, [dk][dv] where it contracts over dv.
 #include "gla_chunk_common.hpp"
 #include "gla_chunk_kernels.hpp"
 
@@ -120,51 +121,96 @@ __global__ __launch_bounds__(C * 4) void chunk_outer_kernel(const float *__restr
     }
 }
 
-// One thread = one dv row x 4 consecutive dk of the transposed state.
+// One thread = a 2x2 patch of the state, one wave = a 16x16 sub-tile (8x8 lanes), one block = a 32x32
+// tile, walked over the chunks in registers.  The running state is written per chunk in BOTH
+// orientations ([dv][dk] for products contracting over dk, [dk][dv] for products contracting over dv);
+// with 8x8 lanes of 2x2 patches every store instruction fills whole 32-byte sectors either way.
+template <typename T> struct Pair;
+template <> struct Pair<__bf16> { typedef bf16x2 type; };
+template <> struct Pair<float> { typedef f32x2 type; };
+
 template <typename T, int D>
 __global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ hin,
                                                          const float *__restrict__ prodT,
                                                          const float *__restrict__ decay,
-                                                         T *__restrict__ states, T *__restrict__ hout,
-                                                         int N, int reverse)
+                                                         T *__restrict__ statesT, T *__restrict__ statesN,
+                                                         T *__restrict__ hout, int N, int reverse)
 {
-    const int idx = blockIdx.x * 256 + threadIdx.x;   // over D * D/4
+    typedef typename Pair<T>::type P2;
+    constexpr int TPD = D / 32;
     const int bh = blockIdx.y;
-    const int dv = idx / (D / 4), dk0 = (idx % (D / 4)) * 4;
-    float X[4];
+    const int tile_v = blockIdx.x / TPD, tile_k = blockIdx.x % TPD;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ti = lane >> 3, tj = lane & 7;
+    const int dv0 = 32 * tile_v + 16 * (wave >> 1) + 2 * ti;
+    const int dk0 = 32 * tile_k + 16 * (wave & 1) + 2 * tj;
+    float X[2][2];   // X[i][j] = S[dk0 + j][dv0 + i]
 #pragma unroll
-    for (int e = 0; e < 4; ++e) X[e] = Elem<T>::load(hin + (int64_t)bh * D * D + (dk0 + e) * D + dv);
-    const float *pp = prodT + (int64_t)bh * N * D * D + dv * D + dk0;
+    for (int j = 0; j < 2; ++j) {
+        P2 t = *reinterpret_cast<const P2 *>(hin + (int64_t)bh * D * D + (dk0 + j) * D + dv0);
+        X[0][j] = (float)t[0];
+        X[1][j] = (float)t[1];
+    }
+    const float *pp = prodT + (int64_t)bh * N * D * D + dv0 * D + dk0;
     const float *dp = decay + (int64_t)bh * N * D + dk0;
-    T *sp = states + (int64_t)bh * N * D * D + dv * D + dk0;
+    const int64_t sbase = (int64_t)bh * N * D * D;
+    auto emit = [&](int n) {
+        if (statesT) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                P2 t;
+                t[0] = X[i][0]; t[1] = X[i][1];
+                *reinterpret_cast<P2 *>(statesT + sbase + (int64_t)n * D * D + (dv0 + i) * D + dk0) = t;
+            }
+        }
+        if (statesN) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                P2 t;
+                t[0] = X[0][j]; t[1] = X[1][j];
+                *reinterpret_cast<P2 *>(statesN + sbase + (int64_t)n * D * D + (dk0 + j) * D + dv0) = t;
+            }
+        }
+    };
     constexpr int U = 4;
     int step = 0;
     for (; step + U <= N; step += U) {
-        f32x4 pv[U], dv4[U];
+        f32x2 pv[U][2], dc[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int n = reverse ? N - 1 - (step + u) : step + u;
-            pv[u] = *reinterpret_cast<const f32x4 *>(pp + (int64_t)n * D * D);
-            dv4[u] = *reinterpret_cast<const f32x4 *>(dp + (int64_t)n * D);
+            pv[u][0] = *reinterpret_cast<const f32x2 *>(pp + (int64_t)n * D * D);
+            pv[u][1] = *reinterpret_cast<const f32x2 *>(pp + (int64_t)n * D * D + D);
+            dc[u] = *reinterpret_cast<const f32x2 *>(dp + (int64_t)n * D);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int n = reverse ? N - 1 - (step + u) : step + u;
-            store_vec<T, 4>(sp + (int64_t)n * D * D, X);
+            emit(n);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) X[e] = dv4[u][e] * X[e] + pv[u][e];
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) X[i][j] = dc[u][j] * X[i][j] + pv[u][i][j];
         }
     }
     for (; step < N; ++step) {
         const int n = reverse ? N - 1 - step : step;
-        f32x4 pv = *reinterpret_cast<const f32x4 *>(pp + (int64_t)n * D * D);
-        f32x4 dd = *reinterpret_cast<const f32x4 *>(dp + (int64_t)n * D);
-        store_vec<T, 4>(sp + (int64_t)n * D * D, X);
+        f32x2 p0 = *reinterpret_cast<const f32x2 *>(pp + (int64_t)n * D * D);
+        f32x2 p1 = *reinterpret_cast<const f32x2 *>(pp + (int64_t)n * D * D + D);
+        f32x2 dc = *reinterpret_cast<const f32x2 *>(dp + (int64_t)n * D);
+        emit(n);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) X[e] = dd[e] * X[e] + pv[e];
+        for (int j = 0; j < 2; ++j) {
+            X[0][j] = dc[j] * X[0][j] + p0[j];
+            X[1][j] = dc[j] * X[1][j] + p1[j];
+        }
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) Elem<T>::store(hout + (int64_t)bh * D * D + (dk0 + e) * D + dv, X[e]);
+    for (int j = 0; j < 2; ++j) {
+        P2 t;
+        t[0] = X[0][j]; t[1] = X[1][j];
+        *reinterpret_cast<P2 *>(hout + (int64_t)bh * D * D + (dk0 + j) * D + dv0) = t;
+    }
 }
 
 template <typename T, int C, int D>
@@ -188,11 +234,11 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
 
 template <typename T, int D>
 int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hin, const float *prodT,
-                      const float *decay, void *states, void *hout)
+                      const float *decay, void *statesT, void *statesN, void *hout)
 {
-    dim3 grid(D * D / 4 / 256, BH), block(256);
+    dim3 grid((D / 32) * (D / 32), BH), block(256);
     hipLaunchKernelGGL((chunk_scan_kernel<T, D>), grid, block, 0, st, (const T *)hin, prodT, decay,
-                       (T *)states, (T *)hout, N, reverse);
+                       (T *)statesT, (T *)statesN, (T *)hout, N, reverse);
     return launch_status();
 }
 
@@ -201,7 +247,7 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hi
                                              const void *, float *, float *);
 #define GLA_INST_SCAN(T, D)                                                                           \
     template int launch_chunk_scan<T, D>(hipStream_t, int, int, int, const void *, const float *,     \
-                                         const float *, void *, void *);
+                                         const float *, void *, void *, void *);
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUTER)
 GLA_INST_SCAN(__bf16, 64)
 GLA_INST_SCAN(__bf16, 128)
