@@ -18,8 +18,10 @@
 
 namespace gla {
 
+// Two tiles and a table fit twice into a CU's LDS; the register budget is held to what lets two
+// workgroups share a CU, so that one loads while the other computes.
 template <typename T, int C, int D, int MODE>
-__global__ __launch_bounds__(C * 4) void chunk_outer_kernel(const float *__restrict__ g,
+__global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C / 32))) void chunk_outer_kernel(const float *__restrict__ g,
                                                             const T *__restrict__ x,
                                                             const T *__restrict__ y,
                                                             float *__restrict__ prodT,
@@ -30,7 +32,8 @@ __global__ __launch_bounds__(C * 4) void chunk_outer_kernel(const float *__restr
     extern __shared__ __align__(16) unsigned char smem[];
     T *Xn = reinterpret_cast<T *>(smem);
     T *Yn = Xn + C * LS;
-    float *rtab = reinterpret_cast<float *>(Yn + C * LS);   // [NB][D]
+    float *rtab = reinterpret_cast<float *>(Yn + C * LS);   // [NB][D] e^{tau_m}
+    float *ttab = rtab + NB * D;                            // [NB][D] tau_m (log2 units)
 
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int r = lane & 15, c = lane >> 4;
@@ -41,27 +44,28 @@ __global__ __launch_bounds__(C * 4) void chunk_outer_kernel(const float *__restr
     const int64_t tok = (int64_t)b * T_len + (int64_t)n * C + 16 * w + r;
     const int64_t rowoff = (tok * H + h) * D;
 
-    float p[NV], s[NV];
+    float p[NV];
     typename FragTypes<T>::d8 yf[KS], xf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const int d0 = 32 * ks + 8 * c;
         f32x8 gg = ld8(g + rowoff + d0);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
+        for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
         yf[ks] = ld8(y + rowoff + d0);
         xf[ks] = ld8(x + rowoff + d0);
     }
-    hier_step<1>(p, s, (r & 1) != 0);
-    hier_step<2>(p, s, (r & 2) != 0);
-    hier_step<4>(p, s, (r & 4) != 0);
-    hier_step<8>(p, s, (r & 8) != 0);
-    if (r == 0) {
+    // p = gate prefix inside the sub-block (log2 units); row 15 holds the sub-block total tau, which
+    // goes to ttab as it is and to rtab as e^{tau}.
+#pragma unroll
+    for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
+    if (r == 15) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             f32x8 t;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p[8 * ks + e] + s[8 * ks + e]);
+            for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p[8 * ks + e]);
+            st8(ttab + w * D + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
             st8(rtab + w * D + 32 * ks + 8 * c, t);
         }
     }
@@ -72,8 +76,14 @@ __global__ __launch_bounds__(C * 4) void chunk_outer_kernel(const float *__restr
     for (int ks = 0; ks < KS; ++ks) {
         const int d0 = 32 * ks + 8 * c;
         float f[8], yv[8];
+        if (MODE == 0) {
+            f32x8 tau = ld8(ttab + w * D + d0);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) f[e] = fast_exp2(MODE == 0 ? s[8 * ks + e] : p[8 * ks + e]);
+            for (int e = 0; e < 8; ++e) f[e] = fast_exp2(tau.v[e] - p[8 * ks + e]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = fast_exp2(p[8 * ks + e]);
+        }
         float all[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) all[e] = 1.f;
@@ -218,7 +228,7 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
                        const void *y, float *prodT, float *decay)
 {
     constexpr int LS = TileGeom<T, D>::kStride;
-    const size_t lds = (size_t)2 * C * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
+    const size_t lds = (size_t)2 * C * LS * sizeof(T) + (size_t)2 * (C / 16) * D * sizeof(float);
     dim3 grid(T_len / C * H, B), block(C * 4);
     if (mode == 0) {
         auto kern = chunk_outer_kernel<T, C, D, 0>;
