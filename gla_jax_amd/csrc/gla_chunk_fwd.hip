@@ -19,24 +19,26 @@
 
 namespace gla {
 
+// Resources: two tiles (keys of all but the last sub-block, values), 32 staged state rows and a table
+// fit twice into a CU's LDS, and the register budget is held to what lets two workgroups share a CU, so
+// that one loads while the other computes.
 template <typename T, int C, int D>
-__global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restrict__ g,
-                                                          const T *__restrict__ v,
-                                                          const T *__restrict__ k,
-                                                          const T *__restrict__ q,
-                                                          const T *__restrict__ states,
-                                                          T *__restrict__ out, int T_len, int H)
+__global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C / 32))) void chunk_out_kernel(
+    const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k, const T *__restrict__ q,
+    const T *__restrict__ states, T *__restrict__ out, int T_len, int H)
 {
-    constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16;
+    constexpr int NB = C / 16, KS = D / 32, NV = D / 4;
     constexpr int LS = TileGeom<T, D>::kStride;
     typedef typename FragTypes<T>::d8 D8;
+    typedef typename FragTypes<T>::t4 T4;
     extern __shared__ __align__(16) unsigned char smem[];
-    T *Kh = reinterpret_cast<T *>(smem);           // [C][LS]  k * exp(tau_J - l_j)
-    T *Vn = Kh + C * LS;                           // [C][LS]  value
-    T *St = Vn + C * LS;                           // [D][LS]  chunk-start state, [dv][dk]
-    float *rtab = reinterpret_cast<float *>(St + D * LS);   // [NB][D] exp(tau_m)
+    T *Vn = reinterpret_cast<T *>(smem);           // [C][LS]       value
+    T *Kh = Vn + C * LS;                           // [C - 16][LS]  k * exp(tau_J - l_j), sub-blocks 0 .. NB-2
+    T *St = Kh + (C - 16) * LS;                    // [32][LS]      32 rows of the chunk-start state [dv][dk]
+    float *rtab = reinterpret_cast<float *>(St + 32 * LS);   // [NB][D] exp(tau_m)
 
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, c = lane >> 4;
     // heads vary fastest over the grid: workgroups that run together touch the same DRAM pages of the
     // [B, T, H, D] arrays (a token's H rows are contiguous)
@@ -47,188 +49,224 @@ __global__ __launch_bounds__(C * 4) void chunk_out_kernel(const float *__restric
     const TrLane<T> L = make_tr_lane<T>(LS);
     const int wrow = 16 * w * LS + L.nat;          // this lane's row of a [token][feature] tile
 
-    float p[NV], s[NV];
-    D8 qf[KS], kf[KS];
+    // 32 rows of the state per slice of the output's features, through registers, one slice ahead
+    constexpr int kPieces = 32 * D / 8;                       // 8-element pieces of a slice
+    constexpr int kPer = (kPieces + C * 4 - 1) / (C * 4);     // pieces per thread
+    D8 pf[kPer];
+    const T *sp = states + (((int64_t)b * H + h) * N + n) * D * D;
+    auto stage_fetch = [&](int slice) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        const int d0 = 32 * ks + 8 * c;
-        f32x8 gg = ld8(g + rowoff + d0);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
-        qf[ks] = ld8(q + rowoff + d0);
-        kf[ks] = ld8(k + rowoff + d0);
-        st8(Vn + wrow + 32 * ks, ld8(v + rowoff + d0));
-    }
-    {
-        const T *sp = states + (((int64_t)b * H + h) * N + n) * D * D;
-        for (int idx = threadIdx.x; idx < D * D / 8; idx += C * 4) {
-            const int row = idx / (D / 8), c8 = (idx % (D / 8)) * 8;
-            st8(St + row * LS + c8, ld8(sp + row * D + c8));
+        for (int u = 0; u < kPer; ++u) {
+            const int idx = threadIdx.x + u * C * 4;
+            if (kPieces % (C * 4) == 0 || idx < kPieces)
+                pf[u] = ld8(sp + (32 * slice + idx / (D / 8)) * D + (idx % (D / 8)) * 8);
         }
-    }
-
-    // ---- gate prefix of the sub-block; can the whole sub-block share ONE anchor? ------------------
-    // p = l_i (inclusive prefix over the 16 rows, log2 units), s = tau - l_i.  The totals travel through
-    // the wave's own row of rtab (same-wave LDS accesses execute in order).
+    };
+    auto stage_store = [&]() {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
-    if (r == 15) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) st8(rtab + w * D + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
-    }
-    asm volatile("" ::: "memory");
-    float span = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        f32x8 tau = ld8(rtab + w * D + 32 * ks + 8 * c);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            s[8 * ks + e] = tau.v[e] - p[8 * ks + e];
-            span = fmaxf(span, fmaxf(fabsf(p[8 * ks + e]), fabsf(s[8 * ks + e])));
+        for (int u = 0; u < kPer; ++u) {
+            const int idx = threadIdx.x + u * C * 4;
+            if (kPieces % (C * 4) == 0 || idx < kPieces) st8(St + (idx / (D / 8)) * LS + (idx % (D / 8)) * 8, pf[u]);
         }
-    }
-    asm volatile("" ::: "memory");
-    const bool one_anchor = wave_all_below(span, kOneAnchorSpan);
+    };
 
     f32x4 accD = {0.f, 0.f, 0.f, 0.f};   // transposed scores of the diagonal sub-block: [j = 4c+e][i = r]
-    if (one_anchor) {
-        // Gates this mild need no recursion: with the anchor at the end of the sub-block,
-        // A_ij = [q_i e^{l_i - tau}] . [k_j e^{tau - l_j}], both factors are finite (at most 2^span) and carry
-        // the same relative rounding as the dyadic form.  The key factor is the operand of the other
-        // sub-blocks as well.
-        f32x4 G = {0.f, 0.f, 0.f, 0.f};
+    float qh[NV];                        // q * exp(l_i), walked down the earlier sub-blocks below
+    {
+        float p[NV];
+        D8 qf[KS], kf[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            float a[8], bq[8];
-            unpack8(qf[ks], a);
-            unpack8(kf[ks], bq);
+            const int d0 = 32 * ks + 8 * c;
+            f32x8 gg = ld8(g + rowoff + d0);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                a[e] *= fast_exp2(-s[8 * ks + e]);
-                bq[e] *= fast_exp2(s[8 * ks + e]);
-            }
-            G = mma_d(pack8<T>(bq), pack8<T>(a), G);
+            for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
+            qf[ks] = ld8(q + rowoff + d0);
+            kf[ks] = ld8(k + rowoff + d0);
+            st8(Vn + wrow + 32 * ks, ld8(v + rowoff + d0));
         }
+        stage_fetch(0);
+
+        // ---- gate prefix of the sub-block; can the whole sub-block share ONE anchor? --------------
+        // p = l_i (inclusive prefix over the 16 rows, log2 units); tau - l_i is rebuilt from the totals, which
+        // travel through the wave's own row of rtab (same-wave LDS accesses execute in order).
 #pragma unroll
-        for (int e = 0; e < 4; ++e) accD[e] = (4 * c + e < r) ? G[e] : 0.f;
-    } else {
-        // ---- the dyadic levels 2, 4, 8, 16 of the reference ------------------------------------------
+        for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
+        if (r == 15) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) st8(rtab + w * D + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
+        }
+        asm volatile("" ::: "memory");
+        float span = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            f32x8 gg = ld8(refetch(g + rowoff) + 32 * ks + 8 * c);
+            f32x8 tau = ld8(rtab + w * D + 32 * ks + 8 * c);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
+            for (int e = 0; e < 8; ++e)
+                span = fmaxf(span, fmaxf(fabsf(p[8 * ks + e]), fabsf(tau.v[e] - p[8 * ks + e])));
         }
-        auto level = [&](auto hc) {
-            constexpr int h_ = decltype(hc)::value;
-            const bool upper = (r & h_) != 0;
+        const bool one_anchor = wave_all_below(span, kOneAnchorSpan);
+
+        if (one_anchor) {
+            // Gates this mild need no recursion: with the anchor at the end of the sub-block,
+            // A_ij = [q_i e^{l_i - tau}] . [k_j e^{tau - l_j}], both factors are finite (at most 2^span) and
+            // carry the same relative rounding as the dyadic form.  The key factor is the operand of the
+            // other sub-blocks as well.
+            float dot = 0.f;
             f32x4 G = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                float a[8], bq[8], x[8];
+                f32x8 tau = ld8(rtab + w * D + 32 * ks + 8 * c);
+                float a[8], bq[8], qo[8];
                 unpack8(qf[ks], a);
                 unpack8(kf[ks], bq);
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    x[e] = (upper ? a[e] : bq[e]) * fast_exp2(upper ? p[8 * ks + e] : s[8 * ks + e]);
-                D8 X = pack8<T>(x);
-                G = mma_d(X, X, G);
+                for (int e = 0; e < 8; ++e) {
+                    const float s = tau.v[e] - p[8 * ks + e];
+                    dot += a[e] * bq[e];
+                    qo[e] = a[e] * fast_exp2(-s);
+                    qh[8 * ks + e] = a[e] * fast_exp2(p[8 * ks + e]);
+                    bq[e] *= fast_exp2(s);
+                }
+                const D8 kh = pack8<T>(bq);
+                if (w < NB - 1) st8(Kh + wrow + 32 * ks, kh);
+                G = mma_d(kh, pack8<T>(qo), G);
+                __builtin_amdgcn_sched_barrier(0);
             }
+            dot = reduce_over_cgroups(dot);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) accD[e] = (4 * c + e < r) ? G[e] : ((4 * c + e == r) ? dot : 0.f);
+            asm volatile("" ::: "memory");
+            if (r == 0) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    f32x8 tau = ld8(rtab + w * D + 32 * ks + 8 * c);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) tau.v[e] = fast_exp2(tau.v[e]);
+                    st8(rtab + w * D + 32 * ks + 8 * c, tau);
+                }
+            }
+        } else {
+            // ---- the dyadic levels 2, 4, 8, 16 of the reference --------------------------------------
+            // At level 2h rows in the upper half of their group carry q e^{prefix over the half}, rows in
+            // the lower half k e^{suffix over the half}; one MFMA of that mixed tile with itself yields every
+            // block of the level.  Walked 32 features at a time (the level's scores add up over the slices)
+            // with the inputs fetched again, to stay inside the register budget on this rare path.
+            f32x4 Gl[4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+            float dot = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                float p8[8], s8[8], a[8], bq[8];
+                {
+                    f32x8 gg = ld8(refetch(g + rowoff) + 32 * ks + 8 * c);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) { p8[e] = gg.v[e] * kLog2e; s8[e] = 0.f; }
+                    unpack8(ld8(refetch(q + rowoff) + 32 * ks + 8 * c), a);
+                    unpack8(ld8(refetch(k + rowoff) + 32 * ks + 8 * c), bq);
+                }
+                auto level = [&](auto hc, auto lc) {
+                    constexpr int h_ = decltype(hc)::value, L_ = decltype(lc)::value;
+                    const bool upper = (r & h_) != 0;
+                    float x[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) x[e] = (upper ? a[e] : bq[e]) * fast_exp2(upper ? p8[e] : s8[e]);
+                    D8 X = pack8<T>(x);
+                    Gl[L_] = mma_d(X, X, Gl[L_]);
+                    hier_step<h_>(p8, s8, upper);
+                };
+                level(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+                level(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
+                level(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
+                level(std::integral_constant<int, 8>{}, std::integral_constant<int, 3>{});
+                // p8 = l_i, s8 = tau - l_i.  Rescaled operands, diagonal, table of exp(tau).
+                if (r == 0) {
+                    f32x8 t;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p8[e] + s8[e]);
+                    st8(rtab + w * D + 32 * ks + 8 * c, t);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    dot += a[e] * bq[e];
+                    qh[8 * ks + e] = a[e] * fast_exp2(p8[e]);
+                    bq[e] *= fast_exp2(s8[e]);
+                }
+                if (w < NB - 1) st8(Kh + wrow + 32 * ks, pack8<T>(bq));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            dot = reduce_over_cgroups(dot);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int j = 4 * c + e;
-                const bool ok = ((j ^ r) < 2 * h_) && upper && !(j & h_);
-                accD[e] += ok ? G[e] : 0.f;
-            }
-            hier_step<h_>(p, s, upper);
-        };
-        level(std::integral_constant<int, 1>{});
-        level(std::integral_constant<int, 2>{});
-        level(std::integral_constant<int, 4>{});
-        level(std::integral_constant<int, 8>{});
-    }
-
-    // p = l_i (inclusive, log2 units), s = tau - l_i.  Rescaled operands, diagonal, table of exp(tau).
-    float qh[NV];
-    {
-        float dot = 0.f;
+                float acc = (j == r) ? dot : 0.f;                  // plain fp32 dot on the diagonal (gla.py:983)
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            float a[8], bq[8], kh[8];
-            unpack8(qf[ks], a);
-            unpack8(kf[ks], bq);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                dot += a[e] * bq[e];
-                qh[8 * ks + e] = a[e] * fast_exp2(p[8 * ks + e]);
-                kh[e] = bq[e] * fast_exp2(s[8 * ks + e]);
-            }
-            st8(Kh + wrow + 32 * ks, pack8<T>(kh));
-        }
-        dot = reduce_over_cgroups(dot);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) accD[e] += (4 * c + e == r) ? dot : 0.f;
-        if (r == 0) {
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                f32x8 t;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p[8 * ks + e] + s[8 * ks + e]);
-                st8(rtab + w * D + 32 * ks + 8 * c, t);
+                for (int l = 0; l < 4; ++l) {
+                    const int h_ = 1 << l;
+                    const bool ok = ((j ^ r) < 2 * h_) && (r & h_) && !(j & h_);
+                    acc += ok ? Gl[l][e] : 0.f;
+                }
+                accD[e] = acc;
             }
         }
     }
+    stage_store();
     __syncthreads();
+    if (KS > 1) stage_fetch(1);
 
-    // ---- earlier sub-blocks J < w, walking the q side down ---------------------------------------
-    f32x4 accT[NB];
+    // ---- earlier sub-blocks J < w, walking the q side down; scores kept as packed MFMA operands ----
+    T4 sc[NB];
 #pragma unroll
     for (int J = NB - 2; J >= 0; --J) {
-        accT[J] = f32x4{0.f, 0.f, 0.f, 0.f};
+        f32x4 a = {0.f, 0.f, 0.f, 0.f};
         if (J < w) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 D8 qb = pack8<T>(qh + 8 * ks);
                 D8 ka = ld8(Kh + L.nat + 16 * J * LS + 32 * ks);
-                accT[J] = mma_d(ka, qb, accT[J]);
+                a = mma_d(ka, qb, a);
                 f32x8 rr = ld8(rtab + J * D + 32 * ks + 8 * c);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) qh[8 * ks + e] *= rr.v[e];
             }
         }
+        sc[J] = pack4<T>(a);
     }
-    accT[NB - 1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    sc[NB - 1] = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
+    const T4 scD = pack4<T>(accD);
+    D8 qb[KS];                           // q * exp(L_i): operand of the state term
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qb[ks] = pack8<T>(qh + 8 * ks);
 
-    // ---- out^T[dv][i]: state term, then the score blocks ----------------------------------------
-    f32x4 acc[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
+    // ---- out^T[dv][i] in slices of 32 output features: state term, then the score blocks ------------
+#pragma unroll 1
     for (int ks = 0; ks < KS; ++ks) {
-        D8 qb = pack8<T>(qh + 8 * ks);   // q * exp(L_i)
+        const int fo = 32 * ks;
+        f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            D8 sa = ld8(St + L.own + own_const(t, 32 * ks, LS));
-            acc[t] = mma_d(sa, qb, acc[t]);
+        for (int k2 = 0; k2 < KS; ++k2) {
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+                acc[tt] = mma_d(ld8(St + L.own + 4 * tt * LS + 32 * k2), qb[k2], acc[tt]);
         }
-    }
 #pragma unroll
-    for (int J = 0; J < NB; ++J) {
-        if (J <= w) {
-            auto b4 = pack4<T>(J == w ? accD : accT[J]);
+        for (int J = 0; J < NB; ++J) {
+            if (J <= w) {
+                const T4 b4 = J == w ? scD : sc[J];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                auto a4 = lds_tr4(Vn + L.k4 + tr_const(16 * J, t, LS), LS);
-                acc[t] = mma_t(a4, b4, acc[t]);
+                for (int tt = 0; tt < 2; ++tt)
+                    acc[tt] = mma_t(lds_tr4(Vn + L.k4 + fo + 4 * tt + 16 * J * LS, LS), b4, acc[tt]);
             }
         }
-    }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
         float o[8];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { o[e] = acc[2 * ks][e]; o[4 + e] = acc[2 * ks + 1][e]; }
-        st8(out + rowoff + 32 * ks + 8 * c, pack8<T>(o));
+        for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
+        st8(out + rowoff + fo + 8 * c, pack8<T>(o));
+        if (ks + 1 < KS) {
+            __syncthreads();             // every wave is done with the staged rows
+            stage_store();
+            __syncthreads();
+            if (ks + 2 < KS) stage_fetch(ks + 2);
+        }
     }
 }
 
@@ -237,7 +275,7 @@ int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, co
                      const void *q, const void *states, void *out)
 {
     constexpr int LS = TileGeom<T, D>::kStride;
-    const size_t lds = (size_t)(2 * C + D) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
+    const size_t lds = (size_t)(2 * C - 16 + 32) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
     auto kern = chunk_out_kernel<T, C, D>;
     if (int e = allow_lds((const void *)kern, lds)) return e;
     dim3 grid(T_len / C * H, B), block(C * 4);
