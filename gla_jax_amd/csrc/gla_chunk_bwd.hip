@@ -131,43 +131,44 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     float dd = 0.f;                      // dA_ii of this lane's row
     D8 vf[KS];                           // this lane's value row (B operand of the dS' product)
     {
+        // Requests go out in the order the results are needed: gates (prefix sums), q and k (rescaled
+        // tiles, scores), then values and dout (their tiles, dA); memory returns them in that order, so the
+        // first steps run while the rest is still on its way.
         float p[NV], s[NV];
         D8 qf[KS], kf[KS], dof[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const int d0 = 32 * ks + 8 * c;
-            f32x8 gg = ld8(g + rowoff + d0);
+            f32x8 gg = ld8(g + rowoff + 32 * ks + 8 * c);
 #pragma unroll
             for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
-            qf[ks] = ld8(q + rowoff + d0);
-            kf[ks] = ld8(k + rowoff + d0);
-            vf[ks] = ld8(v + rowoff + d0);
-            dof[ks] = ld8(dout + rowoff + d0);
-            st8(tV + wrow + 32 * ks, vf[ks]);
-            st8(tO + wrow + 32 * ks, dof[ks]);
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            qf[ks] = ld8(q + rowoff + 32 * ks + 8 * c);
+            kf[ks] = ld8(k + rowoff + 32 * ks + 8 * c);
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            vf[ks] = ld8(v + rowoff + 32 * ks + 8 * c);
+            dof[ks] = ld8(dout + rowoff + 32 * ks + 8 * c);
         }
         stage_fetch(0);
         if (threadIdx.x < D) lbar[threadIdx.x] = 0.f;
 
         // dAn[e] = dA[i = 4c+e][j = r],  dAt[e] = dA[i = r][j = 4c+e]   (dA = dO V^T), own sub-block
         f32x4 dAn = {0.f, 0.f, 0.f, 0.f}, dAt = {0.f, 0.f, 0.f, 0.f};
-        float dot = 0.f;
+        auto own_dA = [&]() {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            dAn = mma_d(dof[ks], vf[ks], dAn);
-            dAt = mma_d(vf[ks], dof[ks], dAt);
-            float a[8], bq[8];
-            unpack8(qf[ks], a);
-            unpack8(kf[ks], bq);
+            for (int ks = 0; ks < KS; ++ks) {
+                st8(tV + wrow + 32 * ks, vf[ks]);
+                st8(tO + wrow + 32 * ks, dof[ks]);
+                dAn = mma_d(dof[ks], vf[ks], dAn);
+                dAt = mma_d(vf[ks], dof[ks], dAt);
+            }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) dot += a[e] * bq[e];
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) dd += (4 * c + e == r) ? dAt[e] : 0.f;
-        dd = reduce_over_cgroups(dd);
-        dot = reduce_over_cgroups(dot);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) Aown[e] = (4 * c + e == r) ? dot : 0.f;   // A_ii = q_i.k_i (gla.py:983)
+            for (int e = 0; e < 4; ++e) dd += (4 * c + e == r) ? dAt[e] : 0.f;
+            dd = reduce_over_cgroups(dd);
+        };
 
         // p = l_i (inclusive prefix over the 16 rows, log2 units), s = tau - l_i; the totals go through
         // the wave's row of ttab (same-wave LDS accesses execute in order) and stay there.
@@ -223,6 +224,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             __builtin_amdgcn_sched_barrier(0);
         };
         if (!one_anchor) {
+            own_dA();
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 f32x8 gg = ld8(refetch(g + rowoff) + 32 * ks + 8 * c);
@@ -248,6 +250,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
         // One anchor (the end of the sub-block): A_ij = [q_i e^{l_i - tau}] . [k_j e^{tau - l_j}]; the key
         // factor is the operand of the other sub-blocks as well.
         f32x4 G = {0.f, 0.f, 0.f, 0.f};
+        float dot = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             float a[8], bq[8], qo[8];
@@ -255,6 +258,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             unpack8(kf[ks], bq);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
+                dot += a[e] * bq[e];
                 qo[e] = a[e] * fast_exp2(-s[8 * ks + e]);
                 a[e] *= fast_exp2(p[8 * ks + e]);
                 bq[e] *= fast_exp2(s[8 * ks + e]);
@@ -264,7 +268,11 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             st8(tK + wrow + 32 * ks, kh);
             if (one_anchor) G = mma_d(pack8<T>(qo), kh, G);
         }
+        dot = reduce_over_cgroups(dot);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) Aown[e] += (4 * c + e == r) ? dot : 0.f;   // A_ii = q_i.k_i (gla.py:983)
         if (one_anchor) {
+            own_dA();
             f32x4 lowT, low;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
