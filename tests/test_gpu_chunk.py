@@ -66,6 +66,33 @@ def test_chunk_strong_decay_and_hard_resets():
     assert_close("hidden_final", to_np(hT), eh, TOL[dtype], stored=dtype)
 
 
+@pytest.mark.parametrize("regime", ["mild", "mixed", "resets"])
+def test_chunk_backward_over_gate_regimes(regime):
+    """Sub-blocks whose gates are mild take the single-anchor path, the others the dyadic recursion; a chunk
+    may hold both kinds.  All five gradients against the oracle in every regime."""
+    from gla_jax_amd import chunk_gla
+    dtype = torch.bfloat16
+    shift = {"mild": 4.0, "mixed": -1.5, "resets": -1.5}[regime]
+    (h0, g, v, k, q), dev = gpu_inputs(1, 256, 2, 128, shift, seed=91, dtype=dtype)
+    g = g.copy()
+    if regime == "resets":
+        g[:, 5::37] = -200.0
+        g[:, 100:104, :, ::2] = -90.0          # only every other feature: the sub-block still takes the recursion
+    dev[1] = to_dev(g, torch.float32)
+    dhT, dout = cotangents(h0, v, 6, dtype)
+    dev = [t.clone().requires_grad_(True) for t in dev]
+    hT, out = chunk_gla(*dev, 128)
+    eh, eo = O.recurrent_gla_naive(h0, g, v, k, q)
+    assert_close("out", to_np(out), eo, TOL[dtype], stored=dtype)
+    assert_close("hidden_final", to_np(hT), eh, TOL[dtype], stored=dtype)
+    loss = (hT.float() * to_dev(dhT, torch.float32)).sum() + (out.float() * to_dev(dout, torch.float32)).sum()
+    grads = torch.autograd.grad(loss, dev)
+    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout)
+    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
+                                grad_kinds(dtype)):
+        assert_close(name, to_np(got), e, TOL[dtype], stored=st)
+
+
 def test_chunk_size_and_concatenation_invariance():
     from gla_jax_amd import chunk_gla
     dtype = torch.float32
