@@ -83,9 +83,7 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
             for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
             qf[ks] = ld8(q + rowoff + d0);
             kf[ks] = ld8(k + rowoff + d0);
-            st8(Vn + wrow + 32 * ks, ld8(v + rowoff + d0));
         }
-        stage_fetch(0);
 
         // ---- gate prefix of the sub-block; can the whole sub-block share ONE anchor? --------------
         // p = l_i (inclusive prefix over the 16 rows, log2 units); tau - l_i is rebuilt from the totals, which
@@ -208,6 +206,16 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
                 accD[e] = acc;
             }
         }
+    }
+    // Values and the first state rows are requested only now: the registers above are free again, and
+    // the other workgroup on the CU covers the wait.
+    {
+        D8 vf[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) vf[ks] = ld8(v + rowoff + 32 * ks + 8 * c);
+        stage_fetch(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) st8(Vn + wrow + 32 * ks, vf[ks]);
     }
     stage_store();
     __syncthreads();
