@@ -49,26 +49,20 @@ template <int N> struct RawVec<__bf16, N> {
     }
 };
 
-// Sum over the 16 lanes that share (lane & 3).
+// Lane l = (a = l >> 4, c = l & 15): the 16 lanes that share `a` are one DPP row, so a sum over c is four
+// cross-lane adds inside the VALU (no trip through the LDS crossbar); every lane of the row gets it.
 __device__ __forceinline__ float reduce_over_c(float x)
-{
-    x += shfl_xor_f32(x, 4);
-    x += shfl_xor_f32(x, 8);
-    x += shfl_xor_f32(x, 16);
-    x += shfl_xor_f32(x, 32);
-    return x;
-}
-// Sum over the 4 lanes that share (lane >> 2).
-__device__ __forceinline__ float reduce_over_a(float x)
 {
     x += dpp_f32<kDppQuadXor1>(x);
     x += dpp_f32<kDppQuadXor2>(x);
+    x += dpp_f32<kDppRowHalfMirror>(x);
+    x += dpp_f32<kDppRowMirror>(x);
     return x;
 }
 
 // ------------------------------------------------------------------------------------------------
-// forward.  Block = DV/16 waves = one (b,h); wave w owns state columns [16w, 16w+16); lane (a = l&3,
-// c = l>>2) owns rows [c*RK, (c+1)*RK) x columns 16w + [4a, 4a+4).
+// forward.  Block = DV/16 waves = one (b,h); wave w owns state columns [16w, 16w+16); lane (a = l>>4,
+// c = l&15) owns rows [c*RK, (c+1)*RK) x columns 16w + [4a, 4a+4).
 // ------------------------------------------------------------------------------------------------
 template <typename T, typename TO, int RK, int U>
 __global__ __launch_bounds__(RK * 64) void recurrent_fwd_kernel(
@@ -78,7 +72,7 @@ __global__ __launch_bounds__(RK * 64) void recurrent_fwd_kernel(
 {
     constexpr int DK = RK * 16, DV = DK;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int a = lane & 3, c = lane >> 2;
+    const int a = lane >> 4, c = lane & 15;
     const int h = blockIdx.x, b = blockIdx.y;
     const int dk0 = c * RK, dv0 = wave * 16 + a * 4;
     const int64_t bh = (int64_t)b * H + h;
@@ -168,7 +162,7 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_dq_kernel(
 {
     constexpr int DV = RV * 16, DK = DV;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int a = lane & 3, c = lane >> 2;
+    const int a = lane >> 4, c = lane & 15;
     const int h = blockIdx.x, b = blockIdx.y;
     const int dk0 = wave * 16 + a * 4, dv0 = c * RV;
     const int64_t bh = (int64_t)b * H + h;
@@ -258,9 +252,9 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_rev_kernel(
     T *__restrict__ dk, int T_len, int H, int reverse)
 {
     constexpr int DV = RV * 16, DK = DV, NW = RV;
-    __shared__ float part[TB * NW * DV];
+    __shared__ float part[TB * NW * 4 * DV];   // [slot][wave][a][dv]: partial dv of 4 state rows each
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int a = lane & 3, c = lane >> 2;
+    const int a = lane >> 4, c = lane & 15;
     const int h = blockIdx.x, b = blockIdx.y;
     const int dk0 = wave * 16 + a * 4, dv0 = c * RV;
     const int64_t bh = (int64_t)b * H + h;
@@ -322,13 +316,7 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_rev_kernel(
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) dkk[i] = reduce_over_c(dkk[i]);
-#pragma unroll
-        for (int j = 0; j < RV; ++j) dvv[j] = reduce_over_a(dvv[j]);
-        if (a == 0) {
-            float *pp = part + ((size_t)slot * NW + wave) * DV + dv0;
-#pragma unroll
-            for (int j = 0; j < RV; ++j) pp[j] = dvv[j];
-        }
+        store_vec<float, RV>(part + (((size_t)slot * NW + wave) * 4 + a) * DV + dv0, dvv);
         float o[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -346,7 +334,7 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_rev_kernel(
         for (int idx = threadIdx.x; idx < count * DV; idx += blockDim.x) {
             int slot = idx / DV, col = idx % DV;
             float s = 0.f;
-            for (int w = 0; w < NW; ++w) s += part[((size_t)slot * NW + w) * DV + col];
+            for (int w = 0; w < NW * 4; ++w) s += part[((size_t)slot * NW * 4 + w) * DV + col];
             int t = phys(first_step - slot);
             Elem<T>::store(dv + offVrow + t * strideV + col, s);
         }
