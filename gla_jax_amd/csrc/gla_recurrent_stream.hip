@@ -1,0 +1,271 @@
+// recurrent_gla forward for bf16 inputs on the matrix cores: one workgroup streams over the sequence of
+// one (batch, head) pair with the [DK,DV] state in fp32 accumulator registers; no hidden state ever
+// touches HBM (gla.py:50-96 keeps the state of a program in registers the same way).
+//
+// The rank-1 updates of C consecutive timesteps are applied together.  With L_t the gate sum from the
+// start of the block of C steps to t and Lend its total,
+//     o_t  = (q_t e^{L_t})^T S_in + sum_{j<=t} A_tj v_j ,        A_tj = sum_d q_td k_jd e^{L_td - L_jd}
+//     S_out = diag(e^{Lend}) S_in + sum_j (k_j e^{Lend - L_j}) v_j^T
+// which is the recurrence S_t = diag(e^{g_t}) S_{t-1} + k_t v_t^T, o_t = S_t^T q_t written out for C steps
+// (gla.py:35-37).  The block is cut into 16-step sub-blocks, one per wave; scores inside a sub-block and
+// the rescaled operands come from subblock_forward (every exponent <= 0, or bounded, see there), pairs
+// of sub-blocks multiply the query side down by e^{tau_m} per step, and the state update is a Horner chain
+// over the sub-blocks: S <- S * e^{tau_J} + V_J^T (k e^{tau_J - l})_J, so nothing is rescaled by a factor
+// above 1; the rescaled keys enter it as bf16 head + remainder, so the update is as exact as the fp32
+// rank-1 updates of the reference.  The state enters the output product as a pair of bf16 numbers (head + remainder, 16 bits of
+// mantissa), so the fp32 state of the reference (gla.py:89) is not rounded where it is used.
+//
+// Steps past the end of the sequence are padded with g = 0, k = v = q = 0 (they leave the state alone and
+// are not stored), so any T works.  `reverse` walks the sequence from its end (gla.py:421-438).
+#include "gla_subblock.hpp"
+#include "gla_recurrent_stream.hpp"
+
+namespace gla {
+
+template <typename TO> struct OutPack;
+template <> struct OutPack<__bf16> {
+    static __device__ __forceinline__ void store(__bf16 *p, const float *o) { st8(p, pack8<__bf16>(o)); }
+};
+template <> struct OutPack<float> {
+    static __device__ __forceinline__ void store(float *p, const float *o) { st8(p, pack8<float>(o)); }
+};
+
+template <typename TO, int C, int D>
+__global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
+    const __bf16 *__restrict__ h0, const float *__restrict__ g, const __bf16 *__restrict__ v,
+    const __bf16 *__restrict__ k, const __bf16 *__restrict__ q, __bf16 *__restrict__ hT,
+    TO *__restrict__ out, int T_len, int H, int reverse)
+{
+    typedef __bf16 T;
+    constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16, RT = NT / NB;
+    static_assert(NT % NB == 0, "every wave owns the same number of state row tiles");
+    constexpr int LS = TileGeom<T, D>::kStride;
+    typedef typename FragTypes<T>::d8 D8;
+    typedef typename FragTypes<T>::t4 T4;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *Vn = reinterpret_cast<T *>(smem);           // [C][LS]  value
+    T *Kh = Vn + C * LS;                           // [C][LS]  k * exp(tau_J - l_j)
+    T *Kl = Kh + C * LS;                           // [C][LS]  what the bf16 rounding of Kh leaves over
+    T *St = Kl + C * LS;                           // [D][LS]  state at the start of the block, [dv][dk]: bf16 head
+    T *Sl = St + D * LS;                           // [D][LS]  ... and the bf16 of what the head leaves over
+    float *rtab = reinterpret_cast<float *>(Sl + D * LS);   // [NB][D] exp(tau_m)
+
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, c = lane >> 4;
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int64_t seq = ((int64_t)b * T_len * H + h) * D;      // element offset of (b, t = 0, h)
+    const int64_t rowstride = (int64_t)H * D;
+    const int64_t bh = (int64_t)b * H + h;
+    const TrLane<T> L = make_tr_lane<T>(LS);
+    const int ptl = plain_tr_lane<T>(LS);
+    const int wrow = 16 * w * LS + L.nat;          // this lane's row of a [token][feature] tile
+    const int N = (T_len + C - 1) / C;
+
+    // state: S[i][nt][e] = state[dk = 16nt + r][dv = 16(w + i NB) + 4c + e]  (accumulator layout of a
+    // (dv x dk) product tile)
+    f32x4 S[RT][NT];
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            float t4[4];
+            load_vec<T, 4>(h0 + bh * D * D + (int64_t)(16 * nt + r) * D + 16 * (w + i * NB) + 4 * c, t4);
+            S[i][nt] = f32x4{t4[0], t4[1], t4[2], t4[3]};
+        }
+    auto publish_state = [&]() {
+#pragma unroll
+        for (int i = 0; i < RT; ++i)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const T hi = (T)S[i][nt][e];
+                    St[(16 * (w + i * NB) + 4 * c + e) * LS + 16 * nt + r] = hi;
+                    Sl[(16 * (w + i * NB) + 4 * c + e) * LS + 16 * nt + r] = (T)(S[i][nt][e] - (float)hi);
+                }
+    };
+    publish_state();
+
+    // inputs of the wave's 16 steps of a block, one block ahead
+    f32x8 gN[KS];
+    D8 qN[KS], kN[KS], vN[KS];
+    bool validN;
+    int64_t rowN;
+    auto fetch = [&](int n) {
+        const int s = n * C + 16 * w + r;                      // logical step
+        validN = s < T_len;
+        const int sc = validN ? s : T_len - 1;
+        rowN = seq + (int64_t)(reverse ? T_len - 1 - sc : sc) * rowstride;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            gN[ks] = ld8(g + rowN + 32 * ks + 8 * c);
+            qN[ks] = ld8(q + rowN + 32 * ks + 8 * c);
+            kN[ks] = ld8(k + rowN + 32 * ks + 8 * c);
+            vN[ks] = ld8(v + rowN + 32 * ks + 8 * c);
+        }
+    };
+    fetch(0);
+
+#pragma unroll 1
+    for (int n = 0; n < N; ++n) {
+        const bool valid = validN;
+        const int64_t row = rowN;
+        f32x4 accD = {0.f, 0.f, 0.f, 0.f};   // transposed scores of the own sub-block: [j = 4c+e][i = r]
+        float qh[NV];                        // q * exp(l_i), walked down the earlier sub-blocks below
+        {
+            float p[NV];
+            D8 qf[KS], kf[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                const D8 z8 = pack8<T>(z);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) p[8 * ks + e] = valid ? gN[ks].v[e] * kLog2e : 0.f;
+                qf[ks] = valid ? qN[ks] : z8;
+                kf[ks] = valid ? kN[ks] : z8;
+                st8(Vn + wrow + 32 * ks, valid ? vN[ks] : z8);
+            }
+            if (n + 1 < N) fetch(n + 1);
+            subblock_forward<T, D, true>(p, qf, kf, g + row, q + row, k + row, valid, rtab + w * D, Kh + wrow, true,
+                                   Kl + wrow, r, c, accD, qh);
+        }
+        __syncthreads();                     // tiles of this block and the published state are in place
+
+        // ---- earlier sub-blocks J < w, walking the q side down; scores kept as packed MFMA operands ----
+        // (operands and scores as bf16 head + remainder: the products keep 16 bits of mantissa)
+        auto split4 = [](f32x4 x, T4 &hi, T4 &lo) {
+            hi = pack4<T>(x);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] -= (float)hi[e];
+            lo = pack4<T>(x);
+        };
+        T4 sc[NB], sl[NB];
+#pragma unroll
+        for (int J = NB - 2; J >= 0; --J) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f};
+            if (J < w) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    D8 qbh, qbl;
+                    split8<T>(qh + 8 * ks, qbh, qbl);
+                    a = mma_d_split(ld8(Kh + L.nat + 16 * J * LS + 32 * ks), ld8(Kl + L.nat + 16 * J * LS + 32 * ks),
+                                    qbh, qbl, a);
+                    f32x8 rr = ld8(rtab + J * D + 32 * ks + 8 * c);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) qh[8 * ks + e] *= rr.v[e];
+                }
+            }
+            split4(a, sc[J], sl[J]);
+        }
+        sc[NB - 1] = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
+        sl[NB - 1] = sc[NB - 1];
+        T4 scD, slD;
+        split4(accD, scD, slD);
+        D8 qb[KS], ql[KS];                   // q * exp(L_i), operand of the state term: bf16 head and remainder
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            float hi[8], lo[8];
+            qb[ks] = pack8<T>(qh + 8 * ks);
+            unpack8(qb[ks], hi);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) lo[e] = qh[8 * ks + e] - hi[e];
+            ql[ks] = pack8<T>(lo);
+        }
+
+        // ---- out^T[dv][i] in slices of 32 output features: state term, then the score blocks --------
+#pragma unroll 1
+        for (int ks = 0; ks < KS; ++ks) {
+            const int fo = 32 * ks;
+            f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+            for (int k2 = 0; k2 < KS; ++k2) {
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    const D8 sh = ld8(St + L.own + (fo + 4 * tt) * LS + 32 * k2);
+                    acc[tt] = mma_d(ld8(Sl + L.own + (fo + 4 * tt) * LS + 32 * k2), qb[k2], acc[tt]);
+                    acc[tt] = mma_d(sh, ql[k2], acc[tt]);
+                    acc[tt] = mma_d(sh, qb[k2], acc[tt]);
+                }
+            }
+#pragma unroll
+            for (int J = 0; J < NB; ++J) {
+                if (J <= w) {
+                    const T4 b4 = J == w ? scD : sc[J], l4 = J == w ? slD : sl[J];
+#pragma unroll
+                    for (int tt = 0; tt < 2; ++tt) {
+                        const T4 va = lds_tr4(Vn + L.k4 + fo + 4 * tt + 16 * J * LS, LS);
+                        acc[tt] = mma_t(va, l4, acc[tt]);
+                        acc[tt] = mma_t(va, b4, acc[tt]);
+                    }
+                }
+            }
+            float o[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
+            if (valid) OutPack<TO>::store(out + row + fo + 8 * c, o);
+        }
+
+        // ---- state update: S <- S e^{tau_J} + V_J^T (k e^{tau_J - l})_J over the sub-blocks in order ------
+#pragma unroll
+        for (int J = 0; J < NB; ++J) {
+            float rr[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) rr[nt] = rtab[J * D + 16 * nt + r];
+#pragma unroll
+            for (int i = 0; i < RT; ++i) {
+                auto va = lds_tr4(Vn + ptl + 16 * J * LS + 16 * (w + i * NB), LS);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) S[i][nt][e] *= rr[nt];
+                    S[i][nt] = mma_t(va, lds_tr4(Kl + ptl + 16 * J * LS + 16 * nt, LS), S[i][nt]);
+                    S[i][nt] = mma_t(va, lds_tr4(Kh + ptl + 16 * J * LS + 16 * nt, LS), S[i][nt]);
+                }
+            }
+        }
+        __syncthreads();                     // every wave is done with the tiles and the old state
+        publish_state();
+    }
+
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            float t4[4] = {S[i][nt][0], S[i][nt][1], S[i][nt][2], S[i][nt][3]};
+            store_vec<T, 4>(hT + bh * D * D + (int64_t)(16 * nt + r) * D + 16 * (w + i * NB) + 4 * c, t4);
+        }
+}
+
+template <typename TO, int C, int D>
+static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, const void *h0, const float *g,
+                      const void *v, const void *k, const void *q, void *hT, void *out)
+{
+    typedef __bf16 T;
+    constexpr int LS = TileGeom<T, D>::kStride;
+    const size_t lds = (size_t)(3 * C + 2 * D) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
+    auto kern = recurrent_stream_fwd_kernel<TO, C, D>;
+    if (int e = allow_lds((const void *)kern, lds)) return e;
+    dim3 grid(H, B), block(C * 4);
+    hipLaunchKernelGGL(kern, grid, block, lds, st, (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,
+                       (T *)hT, (TO *)out, T_len, H, reverse);
+    return launch_status();
+}
+
+template <typename TO>
+int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
+                                const float *g, const void *v, const void *k, const void *q, void *hT,
+                                void *out)
+{
+    if (D == 64) return launch_one<TO, 64, 64>(st, B, T_len, H, reverse, h0, g, v, k, q, hT, out);
+    return GLA_ERR_UNSUPPORTED;
+}
+
+template int launch_recurrent_stream_fwd<__bf16>(hipStream_t, int, int, int, int, int, const void *,
+                                                 const float *, const void *, const void *, const void *,
+                                                 void *, void *);
+template int launch_recurrent_stream_fwd<float>(hipStream_t, int, int, int, int, int, const void *,
+                                                const float *, const void *, const void *, const void *,
+                                                void *, void *);
+
+}  // namespace gla

@@ -1,0 +1,14 @@
+// Launchers of the matrix-core recurrent_gla kernels (bf16 inputs, head dimension 64 or 128).
+#pragma once
+
+#include "gla_common.hpp"
+
+namespace gla {
+
+// TO = element type of `out` (__bf16, or float for the recurrent_gla_naive flavour).
+template <typename TO>
+int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
+                                const float *g, const void *v, const void *k, const void *q, void *hT,
+                                void *out);
+
+}  // namespace gla
