@@ -405,11 +405,18 @@ static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
                       void *dk, void *dq)
 {
     dim3 grid(H, B), block(DK / 16 * 64);
+    // sweep 1 of bf16 data at head dimension 64 runs on the matrix cores
+    const bool stream1 = sizeof(T) == 2 && sizeof(TO) == 2 && DK == 64;
+    if (stream1) {
+        int e = launch_recurrent_stream_dq(st, B, T_len, H, DK, reverse, h0, g, v, k, q, dout, dq, dg);
+        if (e) return e;
+    }
 #define GLA_BWD_CASE(RV_, U_, TB_)                                                                      \
     do {                                                                                                \
-        hipLaunchKernelGGL((recurrent_bwd_dq_kernel<T, TO, RV_, U_>), grid, block, 0, st,               \
-                           (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,                  \
-                           (const TO *)dout, (T *)dq, dg, T_len, H, reverse);                           \
+        if (!stream1)                                                                                   \
+            hipLaunchKernelGGL((recurrent_bwd_dq_kernel<T, TO, RV_, U_>), grid, block, 0, st,           \
+                               (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,              \
+                               (const TO *)dout, (T *)dq, dg, T_len, H, reverse);                       \
         hipLaunchKernelGGL((recurrent_bwd_rev_kernel<T, TO, RV_, TB_>), grid, block, 0, st, g,          \
                            (const T *)v, (const T *)k, (const T *)q, (const T *)hT, (const T *)dhT,     \
                            (const TO *)dout, (T *)dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse);        \

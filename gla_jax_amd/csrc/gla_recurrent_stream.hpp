@@ -11,4 +11,9 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
                                 const float *g, const void *v, const void *k, const void *q, void *hT,
                                 void *out);
 
+// Sweep 1 of the backward (bf16 everywhere): dq, and q*dq in fp32 into `qdq`.
+int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
+                               const float *g, const void *v, const void *k, const void *q, const void *dout,
+                               void *dq, float *qdq);
+
 }  // namespace gla

@@ -1,0 +1,395 @@
+// recurrent_gla backward for bf16 inputs on the matrix cores: the two sweeps of gla.py:271-360 with the
+// rank-1 updates of C consecutive timesteps applied together (see gla_recurrent_stream.hip for the block
+// form of the recurrence).  Neither sweep stores a hidden state:
+//   sweep 1 runs along the forward's direction with the state S in accumulator registers and writes
+//           dq_t = S_t do_t and, in fp32 into the d(log_fgate) buffer, q_t * dq_t;
+//   sweep 2 runs against it with dS in accumulator registers and writes dk_t = dS_t v_t, dv_t = dS_t^T k_t,
+//           dh0, and d(log_fgate)_t = sum_{s>=t} (q_s*dq_s - k_s*dk_s) + sum_v dhT*hT   (gla.py:263).
+// Every product whose operand is a rescaled (hence rounded) quantity takes it as bf16 head + remainder,
+// so the gradients carry fp32-grade products like the vector kernels they replace; this also makes the
+// plain difference q*dq - k*dk accurate enough for the gate gradient.
+//
+// Block form, for query row i of sub-block I and key row j of sub-block J of a block (l = gate prefix in the
+// sub-block, tau_m = sub-block totals, r_m = e^{tau_m}, s = tau - l):
+//   dq_i = e^{l_i} ((((S_in do_i) r_0 + G_0) r_1 + G_1) ... r_{I-1} + G_{I-1}) + e^{-s_i} G_I' + dA_ii k_i
+//          G_J = sum_{j in J} dA_ij (k e^{s})_j,  G_I' the same over j < i of the own sub-block,  dA = dO V^T
+// with the dyadic levels of the reference replacing the G_I' term when the gates of the sub-block are hard.
+#include "gla_subblock.hpp"
+#include "gla_recurrent_stream.hpp"
+
+namespace gla {
+
+namespace {
+
+typedef __bf16 BT;
+
+// One level (half-width H) of the dyadic recursion of a 16-token sub-block on a 32-feature slice: the mixed
+// tile X (upper rows q e^{prefix}, lower rows k e^{suffix}) goes through the wave's scratch, dX = (M + M^T) X
+// with M the level's masked dA block; adds the query part (upper rows) to dq8 and/or the key part (lower
+// rows) to dk8.  p8 / s8 are advanced to the next level.
+template <int H, int XS, bool WANT_Q, bool WANT_K>
+__device__ __forceinline__ void bwd_level(float (&p8)[8], float (&s8)[8], const float (&a)[8], const float (&bq)[8],
+                                          f32x4 dAt, f32x4 dAn, BT *xh, BT *xl, int xnat, int xk4, int r, int c,
+                                          float (&dq8)[8], float (&dk8)[8])
+{
+    typedef FragTypes<BT>::d8 D8;
+    typedef FragTypes<BT>::t4 T4;
+    const bool upper = (r & H) != 0;
+    f32x4 sym;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int o = 4 * c + e;                       // the other row
+        const bool same = (o ^ r) < 2 * H;
+        const bool o_up = (o & H) != 0;
+        sym[e] = (same && upper && !o_up) ? dAt[e] : ((same && o_up && !upper) ? dAn[e] : 0.f);
+    }
+    T4 sh, sl;
+    split4<BT>(sym, sh, sl);
+    float fac[8], x[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        fac[e] = fast_exp2(upper ? p8[e] : s8[e]);
+        x[e] = (upper ? a[e] : bq[e]) * fac[e];
+    }
+    D8 Xh, Xl;
+    split8<BT>(x, Xh, Xl);
+    st8(xh + xnat, Xh);
+    st8(xl + xnat, Xl);
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+        f32x4 dx = {0.f, 0.f, 0.f, 0.f};
+        dx = mma_t_split(lds_tr4(xh + xk4 + 4 * tt, XS), lds_tr4(xl + xk4 + 4 * tt, XS), sh, sl, dx);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float z = dx[e] * fac[4 * tt + e];
+            if (WANT_Q) dq8[4 * tt + e] += upper ? z : 0.f;
+            if (WANT_K) dk8[4 * tt + e] += upper ? 0.f : z;
+        }
+    }
+    asm volatile("" ::: "memory");
+    hier_step<H>(p8, s8, upper);
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------------
+// sweep 1
+// ---------------------------------------------------------------------------------------------------
+template <int C, int D>
+__global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
+    const BT *__restrict__ h0, const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k,
+    const BT *__restrict__ q, const BT *__restrict__ dout, BT *__restrict__ dq, float *__restrict__ qdq,
+    int T_len, int H, int reverse)
+{
+    typedef BT T;
+    constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16, RT = NT / NB;
+    static_assert(NT % NB == 0, "every wave owns the same number of state row tiles");
+    constexpr int LS = TileGeom<T, D>::kStride;
+    constexpr int XS = 32 + 16 / (int)sizeof(T);
+    typedef FragTypes<T>::d8 D8;
+    typedef FragTypes<T>::t4 T4;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *Vn = reinterpret_cast<T *>(smem);           // [C][LS]  value
+    T *Kh = Vn + C * LS;                           // [C][LS]  k * exp(tau_J - l_j), bf16 head
+    T *Kl = Kh + C * LS;                           // [C][LS]  ... and remainder
+    T *Sh = Kl + C * LS;                           // [D][LS]  state at the start of the block, [dk][dv], head
+    T *Sl = Sh + D * LS;                           // [D][LS]  ... and remainder
+    T *xs = Sl + D * LS;                           // [NB][2][16][XS] per-wave scratch (hard gates only)
+    float *rtab = reinterpret_cast<float *>(xs + NB * 2 * 16 * XS);   // [NB][D] exp(tau_m)
+
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, c = lane >> 4;
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int64_t seq = ((int64_t)b * T_len * H + h) * D;
+    const int64_t rowstride = (int64_t)H * D;
+    const int64_t bh = (int64_t)b * H + h;
+    const TrLane<T> L = make_tr_lane<T>(LS);
+    const TrLane<T> Lx = make_tr_lane<T>(XS);
+    const int ptl = plain_tr_lane<T>(LS);
+    const int wrow = 16 * w * LS + L.nat;
+    T *xh = xs + (2 * w) * 16 * XS, *xl = xh + 16 * XS;
+    const int N = (T_len + C - 1) / C;
+
+    // state: S[i][nt][e] = state[dk = 16nt + r][dv = 16(w + i NB) + 4c + e]
+    f32x4 S[RT][NT];
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            float t4[4];
+            load_vec<T, 4>(h0 + bh * D * D + (int64_t)(16 * nt + r) * D + 16 * (w + i * NB) + 4 * c, t4);
+            S[i][nt] = f32x4{t4[0], t4[1], t4[2], t4[3]};
+        }
+    auto publish_state = [&]() {
+#pragma unroll
+        for (int i = 0; i < RT; ++i)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                T4 hi, lo;
+                split4<T>(S[i][nt], hi, lo);
+                const int off = (16 * nt + r) * LS + 16 * (w + i * NB) + 4 * c;
+                *reinterpret_cast<T4 *>(Sh + off) = hi;
+                *reinterpret_cast<T4 *>(Sl + off) = lo;
+            }
+    };
+    publish_state();
+
+    f32x8 gN[KS];
+    D8 qN[KS], kN[KS], vN[KS], dN[KS];
+    bool validN;
+    int64_t rowN;
+    auto fetch = [&](int n) {
+        const int s = n * C + 16 * w + r;
+        validN = s < T_len;
+        const int sc = validN ? s : T_len - 1;
+        rowN = seq + (int64_t)(reverse ? T_len - 1 - sc : sc) * rowstride;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            gN[ks] = ld8(g + rowN + 32 * ks + 8 * c);
+            qN[ks] = ld8(q + rowN + 32 * ks + 8 * c);
+            kN[ks] = ld8(k + rowN + 32 * ks + 8 * c);
+            vN[ks] = ld8(v + rowN + 32 * ks + 8 * c);
+            dN[ks] = ld8(dout + rowN + 32 * ks + 8 * c);
+        }
+    };
+    fetch(0);
+
+#pragma unroll 1
+    for (int n = 0; n < N; ++n) {
+        const bool valid = validN;
+        const int64_t row = rowN;
+        float p[NV], dqo[NV];                // l_i; the own sub-block's part of dq (already scaled)
+        D8 qf[KS], kf[KS], dof[KS];
+        T4 lowTh, lowTl;                     // dA^T of the own sub-block below the diagonal (one anchor)
+        bool one_anchor;
+        {
+            D8 vf[KS];
+            float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            const D8 z8 = pack8<T>(z);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) p[8 * ks + e] = valid ? gN[ks].v[e] * kLog2e : 0.f;
+                qf[ks] = valid ? qN[ks] : z8;
+                kf[ks] = valid ? kN[ks] : z8;
+                vf[ks] = valid ? vN[ks] : z8;
+                dof[ks] = valid ? dN[ks] : z8;
+                st8(Vn + wrow + 32 * ks, vf[ks]);
+            }
+            if (n + 1 < N) fetch(n + 1);
+
+            // dAt[e] = dA[i = r][j = 4c+e], dAn[e] = dA[i = 4c+e][j = r]  (dA = dO V^T: exact products of bf16)
+            f32x4 dAn = {0.f, 0.f, 0.f, 0.f}, dAt = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                dAn = mma_d(dof[ks], vf[ks], dAn);
+                dAt = mma_d(vf[ks], dof[ks], dAt);
+            }
+            float dd = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dd += (4 * c + e == r) ? dAt[e] : 0.f;
+            dd = reduce_over_cgroups(dd);
+
+            // gate prefix, totals through the wave's table row, one anchor or not
+            float *rt = rtab + w * D;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
+            if (r == 15) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) st8(rt + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
+            }
+            asm volatile("" ::: "memory");
+            float span = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                f32x8 tau = ld8(rt + 32 * ks + 8 * c);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    span = fmaxf(span, fmaxf(fabsf(p[8 * ks + e]), fabsf(tau.v[e] - p[8 * ks + e])));
+            }
+            one_anchor = wave_all_below(span, kOneAnchorSpan);
+
+            if (one_anchor) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    f32x8 tau = ld8(rt + 32 * ks + 8 * c);
+                    float bq[8];
+                    unpack8(kf[ks], bq);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        dqo[8 * ks + e] = dd * bq[e];                       // diagonal term (gla.py:1181-1185)
+                        bq[e] *= fast_exp2(tau.v[e] - p[8 * ks + e]);
+                    }
+                    D8 kh, kl;
+                    split8<T>(bq, kh, kl);
+                    st8(Kh + wrow + 32 * ks, kh);
+                    st8(Kl + wrow + 32 * ks, kl);
+                }
+                asm volatile("" ::: "memory");
+                if (r == 0) {
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        f32x8 tau = ld8(rt + 32 * ks + 8 * c);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) tau.v[e] = fast_exp2(tau.v[e]);
+                        st8(rt + 32 * ks + 8 * c, tau);
+                    }
+                }
+                f32x4 lowT;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) lowT[e] = (4 * c + e < r) ? dAt[e] : 0.f;
+                split4<T>(lowT, lowTh, lowTl);
+            } else {
+                // hard gates: the dyadic levels, 32 features at a time, inputs fetched again
+                const float live = valid ? 1.f : 0.f;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    float p8[8], s8[8], a[8], bq[8], dq8[8], dk8[8];
+                    f32x8 gg = ld8(refetch(g + row) + 32 * ks + 8 * c);
+                    unpack8(ld8(refetch(q + row) + 32 * ks + 8 * c), a);
+                    unpack8(ld8(refetch(k + row) + 32 * ks + 8 * c), bq);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        p8[e] = gg.v[e] * kLog2e * live;
+                        s8[e] = 0.f;
+                        a[e] *= live;
+                        bq[e] *= live;
+                        dq8[e] = dd * bq[e];
+                    }
+                    bwd_level<1, XS, true, false>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8);
+                    bwd_level<2, XS, true, false>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8);
+                    bwd_level<4, XS, true, false>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8);
+                    bwd_level<8, XS, true, false>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8);
+                    // p8 = l_i, s8 = tau - l_i
+                    if (r == 0) {
+                        f32x8 t;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p8[e] + s8[e]);
+                        st8(rt + 32 * ks + 8 * c, t);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        p[8 * ks + e] = p8[e];
+                        dqo[8 * ks + e] = dq8[e];
+                        bq[e] *= fast_exp2(s8[e]);
+                    }
+                    D8 kh, kl;
+                    split8<T>(bq, kh, kl);
+                    st8(Kh + wrow + 32 * ks, kh);
+                    st8(Kl + wrow + 32 * ks, kl);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                lowTh = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
+                lowTl = lowTh;
+            }
+        }
+        __syncthreads();                     // tiles of this block and the published state are in place
+
+        // ---- dq chain: state term, then the earlier sub-blocks in ascending order, then the own one --------
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int fo = 32 * ks;
+            f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+            for (int k2 = 0; k2 < KS; ++k2) {
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    acc[tt] = mma_d(ld8(Sl + L.own + (fo + 4 * tt) * LS + 32 * k2), dof[k2], acc[tt]);
+                    acc[tt] = mma_d(ld8(Sh + L.own + (fo + 4 * tt) * LS + 32 * k2), dof[k2], acc[tt]);
+                }
+            }
+#pragma unroll
+            for (int J = 0; J < NB - 1; ++J) {
+                if (J < w) {
+                    // dA^T of the pair: [j][i] = v_j . do_i
+                    f32x4 da = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int k2 = 0; k2 < KS; ++k2)
+                        da = mma_d(ld8(Vn + L.nat + 16 * J * LS + 32 * k2), dof[k2], da);
+                    T4 dah, dal;
+                    split4<T>(da, dah, dal);
+                    f32x8 rr = ld8(rtab + J * D + fo + 8 * c);
+#pragma unroll
+                    for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[tt][e] *= rr.v[4 * tt + e];
+                        acc[tt] = mma_t_split(lds_tr4(Kh + L.k4 + fo + 4 * tt + 16 * J * LS, LS),
+                                              lds_tr4(Kl + L.k4 + fo + 4 * tt + 16 * J * LS, LS), dah, dal, acc[tt]);
+                    }
+                }
+            }
+            f32x4 gq[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+            if (one_anchor) {
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+                    gq[tt] = mma_t_split(lds_tr4(Kh + L.k4 + fo + 4 * tt + 16 * w * LS, LS),
+                                         lds_tr4(Kl + L.k4 + fo + 4 * tt + 16 * w * LS, LS), lowTh, lowTl, gq[tt]);
+            }
+            float o[8], a[8];
+            f32x8 rw = ld8(rtab + w * D + fo + 8 * c);       // e^{tau}: e^{-s} = e^{l} / e^{tau}
+            unpack8(qf[ks], a);
+            f32x8 prod;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float el = fast_exp2(p[8 * ks + e]);
+                const float es = one_anchor ? el * __builtin_amdgcn_rcpf(rw.v[e]) : 0.f;
+                o[e] = el * acc[e >> 2][e & 3] + es * gq[e >> 2][e & 3] + dqo[8 * ks + e];
+                prod.v[e] = a[e] * o[e];
+            }
+            if (valid) {
+                st8(dq + row + fo + 8 * c, pack8<T>(o));
+                st8(qdq + row + fo + 8 * c, prod);
+            }
+        }
+
+        // ---- state update: S <- S e^{tau_J} + V_J^T (k e^{tau_J - l})_J over the sub-blocks in order ------
+#pragma unroll
+        for (int J = 0; J < NB; ++J) {
+            float rr[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) rr[nt] = rtab[J * D + 16 * nt + r];
+#pragma unroll
+            for (int i = 0; i < RT; ++i) {
+                auto va = lds_tr4(Vn + ptl + 16 * J * LS + 16 * (w + i * NB), LS);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) S[i][nt][e] *= rr[nt];
+                    S[i][nt] = mma_t(va, lds_tr4(Kl + ptl + 16 * J * LS + 16 * nt, LS), S[i][nt]);
+                    S[i][nt] = mma_t(va, lds_tr4(Kh + ptl + 16 * J * LS + 16 * nt, LS), S[i][nt]);
+                }
+            }
+        }
+        __syncthreads();
+        publish_state();
+    }
+}
+
+template <int C, int D>
+static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, const void *h0, const float *g,
+                     const void *v, const void *k, const void *q, const void *dout, void *dq, float *qdq)
+{
+    typedef BT T;
+    constexpr int LS = TileGeom<T, D>::kStride;
+    constexpr int XS = 32 + 16 / (int)sizeof(T);
+    const size_t lds = ((size_t)(3 * C + 2 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
+                       (size_t)(C / 16) * D * sizeof(float);
+    auto kern = recurrent_stream_dq_kernel<C, D>;
+    if (int e = allow_lds((const void *)kern, lds)) return e;
+    dim3 grid(H, B), block(C * 4);
+    hipLaunchKernelGGL(kern, grid, block, lds, st, (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,
+                       (const T *)dout, (T *)dq, qdq, T_len, H, reverse);
+    return launch_status();
+}
+
+int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
+                               const float *g, const void *v, const void *k, const void *q, const void *dout,
+                               void *dq, float *qdq)
+{
+    if (D == 64) return launch_dq<64, 64>(st, B, T_len, H, reverse, h0, g, v, k, q, dout, dq, qdq);
+    return GLA_ERR_UNSUPPORTED;
+}
+
+}  // namespace gla

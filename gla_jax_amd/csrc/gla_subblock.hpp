@@ -35,6 +35,22 @@ template <typename D8> __device__ __forceinline__ f32x4 mma_d_split(D8 ah, D8 al
     return mma_d(ah, bh, acc);
 }
 
+// The same for 4 accumulator values (a score block as the B operand of a token contraction).
+template <typename T>
+__device__ __forceinline__ void split4(f32x4 x, typename FragTypes<T>::t4 &hi, typename FragTypes<T>::t4 &lo)
+{
+    hi = pack4<T>(x);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[e] -= (float)hi[e];
+    lo = pack4<T>(x);
+}
+template <typename T4> __device__ __forceinline__ f32x4 mma_t_split(T4 ah, T4 al, T4 bh, T4 bl, f32x4 acc)
+{
+    acc = mma_t(al, bh, acc);
+    acc = mma_t(ah, bl, acc);
+    return mma_t(ah, bh, acc);
+}
+
 // PRECISE: the score products take their operands as head + remainder, for callers that promise fp32
 // arithmetic on bf16 inputs; kl_row must be given then.
 template <typename T, int D, bool PRECISE = false>
