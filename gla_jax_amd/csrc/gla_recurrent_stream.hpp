@@ -16,4 +16,9 @@ int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, i
                                const float *g, const void *v, const void *k, const void *q, const void *dout,
                                void *dq, float *qdq);
 
+// Sweep 2: dk, dv, dh0 and dlog_fgate (`dg` holds q*dq from sweep 1 on entry).
+int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, const float *g,
+                                const void *v, const void *k, const void *q, const void *hT, const void *dhT,
+                                const void *dout, void *dh0, float *dg, void *dv, void *dk);
+
 }  // namespace gla

@@ -26,11 +26,12 @@ typedef __bf16 BT;
 // One level (half-width H) of the dyadic recursion of a 16-token sub-block on a 32-feature slice: the mixed
 // tile X (upper rows q e^{prefix}, lower rows k e^{suffix}) goes through the wave's scratch, dX = (M + M^T) X
 // with M the level's masked dA block; adds the query part (upper rows) to dq8 and/or the key part (lower
-// rows) to dk8.  p8 / s8 are advanced to the next level.
-template <int H, int XS, bool WANT_Q, bool WANT_K>
+// rows) to dk8, and (WANT_G) the slice's share of the level's scores X X^T to G.  p8 / s8 are advanced to
+// the next level.
+template <int H, int XS, bool WANT_Q, bool WANT_K, bool WANT_G = false>
 __device__ __forceinline__ void bwd_level(float (&p8)[8], float (&s8)[8], const float (&a)[8], const float (&bq)[8],
                                           f32x4 dAt, f32x4 dAn, BT *xh, BT *xl, int xnat, int xk4, int r, int c,
-                                          float (&dq8)[8], float (&dk8)[8])
+                                          float (&dq8)[8], float (&dk8)[8], f32x4 *G = nullptr)
 {
     typedef FragTypes<BT>::d8 D8;
     typedef FragTypes<BT>::t4 T4;
@@ -53,6 +54,7 @@ __device__ __forceinline__ void bwd_level(float (&p8)[8], float (&s8)[8], const 
     }
     D8 Xh, Xl;
     split8<BT>(x, Xh, Xl);
+    if (WANT_G) *G = mma_d_split(Xh, Xl, Xh, Xl, *G);
     st8(xh + xnat, Xh);
     st8(xl + xnat, Xl);
     asm volatile("" ::: "memory");
@@ -367,6 +369,443 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// sweep 2: against the forward's direction, dS in accumulator registers.  For key row j of sub-block J:
+//   dv_j = sum_{i >= j} A_ij do_i + dS'^T (k e^{Lend - L})_j
+//   dk_j = e^{s_j} ((((dS' v_j) r_{NB-1} + H_{NB-1}) r_{NB-2} + ...) r_{J+1} + H_{J+1}) + e^{s_j} H_J' + dA_jj q_j
+//          H_I = sum_{i in I} dA_ij (q e^{l})_i,  H_J' = sum_{i > j, own sub-block} dA_ij q_i e^{-s_i}
+//   dS_in = diag(e^{Lend}) dS' + sum_i (q e^{L})_i do_i^T     (a Horner chain over the sub-blocks, last first)
+// dS' is the gradient w.r.t. the state after the block.
+// ---------------------------------------------------------------------------------------------------
+template <int C, int D>
+__global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
+    const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k, const BT *__restrict__ q,
+    const BT *__restrict__ hT, const BT *__restrict__ dhT, const BT *__restrict__ dout, BT *__restrict__ dh0,
+    float *__restrict__ dg, BT *__restrict__ dv, BT *__restrict__ dk, int T_len, int H, int reverse)
+{
+    typedef BT T;
+    constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16, RT = NT / NB;
+    static_assert(NT % NB == 0, "every wave owns the same number of state row tiles");
+    constexpr int LS = TileGeom<T, D>::kStride;
+    constexpr int XS = 32 + 16 / (int)sizeof(T);
+    typedef FragTypes<T>::d8 D8;
+    typedef FragTypes<T>::t4 T4;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *tO = reinterpret_cast<T *>(smem);           // [C][LS]  dout
+    T *Qh = tO + C * LS;                           // [C][LS]  q * exp(l_i), bf16 head
+    T *Ql = Qh + C * LS;                           // [C][LS]  ... and remainder
+    T *DNh = Ql + C * LS;                          // [D][LS]  dS' as [dk][dv], head / remainder
+    T *DNl = DNh + D * LS;
+    T *DTh = DNl + D * LS;                         // [D][LS]  dS' as [dv][dk], head / remainder
+    T *DTl = DTh + D * LS;
+    T *xs = DTl + D * LS;                          // [NB][2][16][XS] per-wave scratch
+    float *rtab = reinterpret_cast<float *>(xs + NB * 2 * 16 * XS);   // [NB][D] exp(tau_m)
+    float *dltab = rtab + NB * D;                  // [NB][D] sub-block sums of q*dq - k*dk
+    float *fintab = dltab + NB * D;                // [D] sum_v dhT * hT
+
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, c = lane >> 4;
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int64_t seq = ((int64_t)b * T_len * H + h) * D;
+    const int64_t rowstride = (int64_t)H * D;
+    const int64_t bh = (int64_t)b * H + h;
+    const TrLane<T> L = make_tr_lane<T>(LS);
+    const TrLane<T> Lx = make_tr_lane<T>(XS);
+    const int ptl = plain_tr_lane<T>(LS);
+    const int wrow = 16 * w * LS + L.nat;
+    T *xh = xs + (2 * w) * 16 * XS, *xl = xh + 16 * XS;
+    const int N = (T_len + C - 1) / C;
+
+    // dS: DS[i][nt][e] = dS[dk = 16(w + i NB) + 4c + e][dv = 16nt + r]
+    f32x4 DS[RT][NT];
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                DS[i][nt][e] = (float)dhT[bh * D * D + (int64_t)(16 * (w + i * NB) + 4 * c + e) * D + 16 * nt + r];
+    auto publish = [&]() {
+#pragma unroll
+        for (int i = 0; i < RT; ++i)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                T4 hi, lo;
+                split4<T>(DS[i][nt], hi, lo);
+                const int dk0 = 16 * (w + i * NB) + 4 * c, dvc = 16 * nt + r;
+                *reinterpret_cast<T4 *>(DTh + dvc * LS + dk0) = hi;
+                *reinterpret_cast<T4 *>(DTl + dvc * LS + dk0) = lo;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    DNh[(dk0 + e) * LS + dvc] = hi[e];
+                    DNl[(dk0 + e) * LS + dvc] = lo[e];
+                }
+            }
+    };
+    publish();
+    for (int d = threadIdx.x; d < D; d += C * 4) {
+        float s = 0.f;
+        for (int j = 0; j < D; ++j) s += (float)dhT[bh * D * D + d * D + j] * (float)hT[bh * D * D + d * D + j];
+        fintab[d] = s;
+    }
+    float run[NV];                           // sum over the later blocks of q*dq - k*dk, this lane's features
+#pragma unroll
+    for (int i = 0; i < NV; ++i) run[i] = 0.f;
+
+    f32x8 gN[KS], wN[KS];
+    D8 qN[KS], kN[KS], vN[KS], dN[KS];
+    bool validN;
+    int64_t rowN;
+    auto fetch = [&](int n) {
+        const int s = n * C + 16 * w + r;
+        validN = s < T_len;
+        const int sc = validN ? s : T_len - 1;
+        rowN = seq + (int64_t)(reverse ? T_len - 1 - sc : sc) * rowstride;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            gN[ks] = ld8(g + rowN + 32 * ks + 8 * c);
+            wN[ks] = ld8(dg + rowN + 32 * ks + 8 * c);
+            qN[ks] = ld8(q + rowN + 32 * ks + 8 * c);
+            kN[ks] = ld8(k + rowN + 32 * ks + 8 * c);
+            vN[ks] = ld8(v + rowN + 32 * ks + 8 * c);
+            dN[ks] = ld8(dout + rowN + 32 * ks + 8 * c);
+        }
+    };
+    fetch(N - 1);
+
+#pragma unroll 1
+    for (int n = N - 1; n >= 0; --n) {
+        const bool valid = validN;
+        const int64_t row = rowN;
+        float sv[NV], dko[NV], kt[NV], qdq[NV];  // tau - l_i; own sub-block's part of dk; k e^{s}; q*dq
+        D8 qf[KS], kf[KS], vf[KS], dof[KS];
+        f32x4 Aown = {0.f, 0.f, 0.f, 0.f};       // scores A[i = 4c+e][j = r] of the own sub-block
+        T4 lowh, lowl;                           // dA of the own sub-block below the diagonal (one anchor)
+        f32x4 dAn = {0.f, 0.f, 0.f, 0.f}, dAt = {0.f, 0.f, 0.f, 0.f};
+        bool one_anchor;
+        float dd = 0.f;
+        {
+            float p[NV];
+            float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            const D8 z8 = pack8<T>(z);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    p[8 * ks + e] = valid ? gN[ks].v[e] * kLog2e : 0.f;
+                    qdq[8 * ks + e] = valid ? wN[ks].v[e] : 0.f;
+                }
+                qf[ks] = valid ? qN[ks] : z8;
+                kf[ks] = valid ? kN[ks] : z8;
+                vf[ks] = valid ? vN[ks] : z8;
+                dof[ks] = valid ? dN[ks] : z8;
+                st8(tO + wrow + 32 * ks, dof[ks]);
+            }
+            if (n > 0) fetch(n - 1);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                dAn = mma_d(dof[ks], vf[ks], dAn);
+                dAt = mma_d(vf[ks], dof[ks], dAt);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dd += (4 * c + e == r) ? dAt[e] : 0.f;
+            dd = reduce_over_cgroups(dd);
+
+            float *rt = rtab + w * D;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
+            if (r == 15) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) st8(rt + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
+            }
+            asm volatile("" ::: "memory");
+            float span = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                f32x8 tau = ld8(rt + 32 * ks + 8 * c);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    sv[8 * ks + e] = tau.v[e] - p[8 * ks + e];
+                    span = fmaxf(span, fmaxf(fabsf(p[8 * ks + e]), fabsf(sv[8 * ks + e])));
+                }
+            }
+            one_anchor = wave_all_below(span, kOneAnchorSpan);
+
+            float dot = 0.f;
+            if (one_anchor) {
+                asm volatile("" ::: "memory");
+                if (r == 0) {
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        f32x8 tau = ld8(rt + 32 * ks + 8 * c);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) tau.v[e] = fast_exp2(tau.v[e]);
+                        st8(rt + 32 * ks + 8 * c, tau);
+                    }
+                }
+                f32x4 low;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) low[e] = (4 * c + e > r) ? dAn[e] : 0.f;
+                split4<T>(low, lowh, lowl);
+                f32x4 G = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    float a[8], bq[8], qo[8], qe[8];
+                    unpack8(qf[ks], a);
+                    unpack8(kf[ks], bq);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        dot += a[e] * bq[e];
+                        dko[8 * ks + e] = dd * a[e];
+                        qo[e] = a[e] * fast_exp2(-sv[8 * ks + e]);
+                        qe[e] = a[e] * fast_exp2(p[8 * ks + e]);
+                        kt[8 * ks + e] = bq[e] * fast_exp2(sv[8 * ks + e]);
+                    }
+                    D8 h8, l8, oh, ol, kh, kl;
+                    split8<T>(qe, h8, l8);
+                    st8(Qh + wrow + 32 * ks, h8);
+                    st8(Ql + wrow + 32 * ks, l8);
+                    split8<T>(qo, oh, ol);
+                    split8<T>(kt + 8 * ks, kh, kl);
+                    G = mma_d_split(oh, ol, kh, kl, G);
+                    // own link of dk: H'^T[dk][j] = sum_{i > j} (q e^{-s})_i[dk] dA_ij, through the wave's scratch
+                    st8(xh + Lx.nat, oh);
+                    st8(xl + Lx.nat, ol);
+                    asm volatile("" ::: "memory");
+#pragma unroll
+                    for (int tt = 0; tt < 2; ++tt) {
+                        f32x4 hk = {0.f, 0.f, 0.f, 0.f};
+                        hk = mma_t_split(lds_tr4(xh + Lx.k4 + 4 * tt, XS), lds_tr4(xl + Lx.k4 + 4 * tt, XS), lowh, lowl,
+                                         hk);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            dko[8 * ks + 4 * tt + e] += hk[e] * fast_exp2(sv[8 * ks + 4 * tt + e]);
+                    }
+                    asm volatile("" ::: "memory");
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) Aown[e] = (4 * c + e > r) ? G[e] : 0.f;
+            } else {
+                const float live = valid ? 1.f : 0.f;
+                f32x4 Gl[4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    float p8[8], s8[8], a[8], bq[8], dq8[8], dk8[8];
+                    f32x8 gg = ld8(refetch(g + row) + 32 * ks + 8 * c);
+                    unpack8(ld8(refetch(q + row) + 32 * ks + 8 * c), a);
+                    unpack8(ld8(refetch(k + row) + 32 * ks + 8 * c), bq);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        p8[e] = gg.v[e] * kLog2e * live;
+                        s8[e] = 0.f;
+                        a[e] *= live;
+                        bq[e] *= live;
+                        dk8[e] = dd * a[e];
+                        dot += a[e] * bq[e];
+                    }
+                    bwd_level<1, XS, false, true, true>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8, &Gl[0]);
+                    bwd_level<2, XS, false, true, true>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8, &Gl[1]);
+                    bwd_level<4, XS, false, true, true>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8, &Gl[2]);
+                    bwd_level<8, XS, false, true, true>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8, &Gl[3]);
+                    if (r == 0) {
+                        f32x8 t;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p8[e] + s8[e]);
+                        st8(rt + 32 * ks + 8 * c, t);
+                    }
+                    float qe[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        sv[8 * ks + e] = s8[e];
+                        dko[8 * ks + e] = dk8[e];
+                        qe[e] = a[e] * fast_exp2(p8[e]);
+                        kt[8 * ks + e] = bq[e] * fast_exp2(s8[e]);
+                    }
+                    D8 h8, l8;
+                    split8<T>(qe, h8, l8);
+                    st8(Qh + wrow + 32 * ks, h8);
+                    st8(Ql + wrow + 32 * ks, l8);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int o = 4 * c + e;
+                    float acc = 0.f;
+#pragma unroll
+                    for (int l = 0; l < 4; ++l) {
+                        const int h_ = 1 << l;
+                        const bool ok = ((o ^ r) < 2 * h_) && (o & h_) && !(r & h_);
+                        acc += ok ? Gl[l][e] : 0.f;
+                    }
+                    Aown[e] = acc;
+                }
+                lowh = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
+                lowl = lowh;
+            }
+            dot = reduce_over_cgroups(dot);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) Aown[e] += (4 * c + e == r) ? dot : 0.f;   // A_ii = q_i.k_i (gla.py:983)
+        }
+        __syncthreads();                     // tiles of this block and the published dS' are in place
+
+        // ---- score blocks of the later sub-blocks: A_Ij (key side walked up by r_I) and dA_Ij ----------
+        T4 Ach[NB], Acl[NB], dAh[NB], dAl[NB];
+        D8 Kth[KS], Ktl[KS];                 // k e^{Lend - L_j}, head and remainder
+        {
+            float kch[NV];
+#pragma unroll
+            for (int i = 0; i < NV; ++i) kch[i] = kt[i];
+#pragma unroll
+            for (int I = 1; I < NB; ++I) {
+                Ach[I] = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
+                Acl[I] = Ach[I];
+                dAh[I] = Ach[I];
+                dAl[I] = Ach[I];
+                if (I > w) {
+                    f32x4 a = {0.f, 0.f, 0.f, 0.f}, da = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        D8 kh, kl;
+                        split8<T>(kch + 8 * ks, kh, kl);
+                        a = mma_d_split(ld8(Qh + L.nat + 16 * I * LS + 32 * ks), ld8(Ql + L.nat + 16 * I * LS + 32 * ks),
+                                        kh, kl, a);
+                        da = mma_d(ld8(tO + L.nat + 16 * I * LS + 32 * ks), vf[ks], da);
+                        f32x8 rr = ld8(rtab + I * D + 32 * ks + 8 * c);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) kch[8 * ks + e] *= rr.v[e];
+                    }
+                    split4<T>(a, Ach[I], Acl[I]);
+                    split4<T>(da, dAh[I], dAl[I]);
+                }
+            }
+            split4<T>(Aown, Ach[0], Acl[0]);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) split8<T>(kch + 8 * ks, Kth[ks], Ktl[ks]);
+        }
+
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int fo = 32 * ks;
+            // -- dv slice: dS'^T K~ first, then the own and the later sub-blocks
+            {
+                f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+                for (int k2 = 0; k2 < KS; ++k2) {
+#pragma unroll
+                    for (int tt = 0; tt < 2; ++tt)
+                        acc[tt] = mma_d_split(ld8(DTh + L.own + (fo + 4 * tt) * LS + 32 * k2),
+                                              ld8(DTl + L.own + (fo + 4 * tt) * LS + 32 * k2), Kth[k2], Ktl[k2], acc[tt]);
+                }
+#pragma unroll
+                for (int I = 0; I < NB; ++I) {
+                    if (I >= w) {
+                        const T4 bh4 = I == w ? Ach[0] : Ach[I], bl4 = I == w ? Acl[0] : Acl[I];
+#pragma unroll
+                        for (int tt = 0; tt < 2; ++tt) {
+                            const T4 oa = lds_tr4(tO + L.k4 + fo + 4 * tt + 16 * I * LS, LS);
+                            acc[tt] = mma_t(oa, bl4, acc[tt]);
+                            acc[tt] = mma_t(oa, bh4, acc[tt]);
+                        }
+                    }
+                }
+                float o[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
+                if (valid) st8(dv + row + fo + 8 * c, pack8<T>(o));
+            }
+            // -- dk slice: dS' v first, then the later sub-blocks in descending order
+            {
+                f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+                for (int k2 = 0; k2 < KS; ++k2) {
+#pragma unroll
+                    for (int tt = 0; tt < 2; ++tt) {
+                        acc[tt] = mma_d(ld8(DNl + L.own + (fo + 4 * tt) * LS + 32 * k2), vf[k2], acc[tt]);
+                        acc[tt] = mma_d(ld8(DNh + L.own + (fo + 4 * tt) * LS + 32 * k2), vf[k2], acc[tt]);
+                    }
+                }
+#pragma unroll
+                for (int I = NB - 1; I >= 1; --I) {
+                    if (I > w) {
+                        f32x8 rr = ld8(rtab + I * D + fo + 8 * c);
+#pragma unroll
+                        for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[tt][e] *= rr.v[4 * tt + e];
+                            acc[tt] = mma_t_split(lds_tr4(Qh + L.k4 + fo + 4 * tt + 16 * I * LS, LS),
+                                                  lds_tr4(Ql + L.k4 + fo + 4 * tt + 16 * I * LS, LS), dAh[I], dAl[I],
+                                                  acc[tt]);
+                        }
+                    }
+                }
+                float o[8], kk[8];
+                unpack8(kf[ks], kk);
+                f32x8 sfx;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    o[e] = fast_exp2(sv[8 * ks + e]) * acc[e >> 2][e & 3] + dko[8 * ks + e];
+                    // q*dq - k*dk of the row, then its reverse running sum inside the sub-block
+                    sfx.v[e] = suffix_sum_rows(qdq[8 * ks + e] - kk[e] * o[e]);
+                    qdq[8 * ks + e] = sfx.v[e];
+                }
+                if (valid) st8(dk + row + fo + 8 * c, pack8<T>(o));
+                if (r == 0) st8(dltab + w * D + fo + 8 * c, sfx);
+            }
+        }
+
+        // ---- dS <- dS r_I + (q e^{l})_I^T dO_I over the sub-blocks, last first ---------------------------
+#pragma unroll
+        for (int I = NB - 1; I >= 0; --I) {
+#pragma unroll
+            for (int i = 0; i < RT; ++i) {
+                const f32x4 rr = *reinterpret_cast<const f32x4 *>(rtab + I * D + 16 * (w + i * NB) + 4 * c);
+                const T4 qah = lds_tr4(Qh + ptl + 16 * I * LS + 16 * (w + i * NB), LS);
+                const T4 qal = lds_tr4(Ql + ptl + 16 * I * LS + 16 * (w + i * NB), LS);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) DS[i][nt][e] *= rr[e];
+                    const T4 ob = lds_tr4(tO + ptl + 16 * I * LS + 16 * nt, LS);
+                    DS[i][nt] = mma_t(qal, ob, DS[i][nt]);
+                    DS[i][nt] = mma_t(qah, ob, DS[i][nt]);
+                }
+            }
+        }
+        __syncthreads();                     // sub-block sums complete; every wave is done with the tiles
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            f32x8 o = ld8(fintab + 32 * ks + 8 * c), tot;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                o.v[e] += qdq[8 * ks + e] + run[8 * ks + e];
+                tot.v[e] = 0.f;
+            }
+#pragma unroll
+            for (int m = 0; m < NB; ++m) {
+                f32x8 t = ld8(dltab + m * D + 32 * ks + 8 * c);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    o.v[e] += m > w ? t.v[e] : 0.f;
+                    tot.v[e] += t.v[e];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) run[8 * ks + e] += tot.v[e];
+            if (valid) st8(dg + row + 32 * ks + 8 * c, o);
+        }
+        publish();
+    }
+
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                dh0[bh * D * D + (int64_t)(16 * (w + i * NB) + 4 * c + e) * D + 16 * nt + r] = (T)DS[i][nt][e];
+}
+
 template <int C, int D>
 static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, const void *h0, const float *g,
                      const void *v, const void *k, const void *q, const void *dout, void *dq, float *qdq)
@@ -382,6 +821,32 @@ static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, const
     hipLaunchKernelGGL(kern, grid, block, lds, st, (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,
                        (const T *)dout, (T *)dq, qdq, T_len, H, reverse);
     return launch_status();
+}
+
+template <int C, int D>
+static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, const float *g, const void *v,
+                      const void *k, const void *q, const void *hT, const void *dhT, const void *dout, void *dh0,
+                      float *dg, void *dv, void *dk)
+{
+    typedef BT T;
+    constexpr int LS = TileGeom<T, D>::kStride;
+    constexpr int XS = 32 + 16 / (int)sizeof(T);
+    const size_t lds = ((size_t)(3 * C + 4 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
+                       (size_t)(2 * (C / 16) + 1) * D * sizeof(float);
+    auto kern = recurrent_stream_rev_kernel<C, D>;
+    if (int e = allow_lds((const void *)kern, lds)) return e;
+    dim3 grid(H, B), block(C * 4);
+    hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q, (const T *)hT,
+                       (const T *)dhT, (const T *)dout, (T *)dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse);
+    return launch_status();
+}
+
+int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, const float *g,
+                                const void *v, const void *k, const void *q, const void *hT, const void *dhT,
+                                const void *dout, void *dh0, float *dg, void *dv, void *dk)
+{
+    if (D == 64) return launch_rev<64, 64>(st, B, T_len, H, reverse, g, v, k, q, hT, dhT, dout, dh0, dg, dv, dk);
+    return GLA_ERR_UNSUPPORTED;
 }
 
 int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
