@@ -39,6 +39,31 @@ def test_recurrent_gla_matches_oracle(dtype, B, T, H, D, reverse):
         assert_close(name, to_np(got), e, tol, stored=st)
 
 
+@pytest.mark.parametrize("reverse", [False, True])
+@pytest.mark.parametrize("T", [64, 200, 333])
+def test_recurrent_matrix_core_path_over_gate_regimes(T, reverse):
+    """bf16 at D=64 runs 64 steps per iteration on the matrix cores: sequences that are not a multiple of
+    64 (padded steps), mild gates (one anchor per 16 steps) and hard ones (resets, the dyadic levels) in
+    the same sequence, both directions, forward and all gradients."""
+    from gla_jax_amd import recurrent_gla
+    dtype = torch.bfloat16
+    (h0, g, v, k, q), dev = gpu_inputs(2, T, 2, 64, 1.0, seed=T + 7, dtype=dtype)
+    g = g.copy()
+    g[:, 5::37] = -200.0                       # hard resets at scattered positions
+    g[:, T // 2:T // 2 + 4, :, ::2] = -60.0    # a hard stretch on every other feature
+    dev[1] = to_dev(g, torch.float32)
+    dhT, dout = cotangents(h0, v, 2, dtype)
+    hT, out, grads = run_fwd_bwd(recurrent_gla, dev, to_dev(dhT, dtype), to_dev(dout, dtype), dtype,
+                                 reverse=reverse)
+    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=reverse)
+    tol = TOL[dtype]
+    assert_close("out", to_np(out), exp[6], tol, stored=dtype)
+    assert_close("hidden_final", to_np(hT), exp[5], tol, stored=dtype)
+    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
+                                grad_kinds(dtype)):
+        assert_close(name, to_np(got), e, tol, stored=st)
+
+
 def test_recurrent_gla_naive_returns_fp32_out():
     from gla_jax_amd import recurrent_gla_naive
     dtype = torch.bfloat16
