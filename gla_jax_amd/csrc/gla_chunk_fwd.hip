@@ -14,7 +14,7 @@
 //   * the diagonal is the plain fp32 dot q_i.k_i (gla.py:983).
 // Scores are produced transposed (key token x query token) so that the accumulator registers are
 // directly the B operand of the (feature x token) product with V.
-#include "gla_chunk_common.hpp"
+#include "gla_subblock.hpp"
 #include "gla_chunk_kernels.hpp"
 
 namespace gla {
@@ -85,127 +85,8 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
             kf[ks] = ld8(k + rowoff + d0);
         }
 
-        // ---- gate prefix of the sub-block; can the whole sub-block share ONE anchor? --------------
-        // p = l_i (inclusive prefix over the 16 rows, log2 units); tau - l_i is rebuilt from the totals, which
-        // travel through the wave's own row of rtab (same-wave LDS accesses execute in order).
-#pragma unroll
-        for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
-        if (r == 15) {
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) st8(rtab + w * D + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
-        }
-        asm volatile("" ::: "memory");
-        float span = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            f32x8 tau = ld8(rtab + w * D + 32 * ks + 8 * c);
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                span = fmaxf(span, fmaxf(fabsf(p[8 * ks + e]), fabsf(tau.v[e] - p[8 * ks + e])));
-        }
-        const bool one_anchor = wave_all_below(span, kOneAnchorSpan);
-
-        if (one_anchor) {
-            // Gates this mild need no recursion: with the anchor at the end of the sub-block,
-            // A_ij = [q_i e^{l_i - tau}] . [k_j e^{tau - l_j}], both factors are finite (at most 2^span) and
-            // carry the same relative rounding as the dyadic form.  The key factor is the operand of the
-            // other sub-blocks as well.
-            float dot = 0.f;
-            f32x4 G = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                f32x8 tau = ld8(rtab + w * D + 32 * ks + 8 * c);
-                float a[8], bq[8], qo[8];
-                unpack8(qf[ks], a);
-                unpack8(kf[ks], bq);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float s = tau.v[e] - p[8 * ks + e];
-                    dot += a[e] * bq[e];
-                    qo[e] = a[e] * fast_exp2(-s);
-                    qh[8 * ks + e] = a[e] * fast_exp2(p[8 * ks + e]);
-                    bq[e] *= fast_exp2(s);
-                }
-                const D8 kh = pack8<T>(bq);
-                if (w < NB - 1) st8(Kh + wrow + 32 * ks, kh);
-                G = mma_d(kh, pack8<T>(qo), G);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            dot = reduce_over_cgroups(dot);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) accD[e] = (4 * c + e < r) ? G[e] : ((4 * c + e == r) ? dot : 0.f);
-            asm volatile("" ::: "memory");
-            if (r == 0) {
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    f32x8 tau = ld8(rtab + w * D + 32 * ks + 8 * c);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) tau.v[e] = fast_exp2(tau.v[e]);
-                    st8(rtab + w * D + 32 * ks + 8 * c, tau);
-                }
-            }
-        } else {
-            // ---- the dyadic levels 2, 4, 8, 16 of the reference --------------------------------------
-            // At level 2h rows in the upper half of their group carry q e^{prefix over the half}, rows in
-            // the lower half k e^{suffix over the half}; one MFMA of that mixed tile with itself yields every
-            // block of the level.  Walked 32 features at a time (the level's scores add up over the slices)
-            // with the inputs fetched again, to stay inside the register budget on this rare path.
-            f32x4 Gl[4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-            float dot = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                float p8[8], s8[8], a[8], bq[8];
-                {
-                    f32x8 gg = ld8(refetch(g + rowoff) + 32 * ks + 8 * c);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) { p8[e] = gg.v[e] * kLog2e; s8[e] = 0.f; }
-                    unpack8(ld8(refetch(q + rowoff) + 32 * ks + 8 * c), a);
-                    unpack8(ld8(refetch(k + rowoff) + 32 * ks + 8 * c), bq);
-                }
-                auto level = [&](auto hc, auto lc) {
-                    constexpr int h_ = decltype(hc)::value, L_ = decltype(lc)::value;
-                    const bool upper = (r & h_) != 0;
-                    float x[8];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) x[e] = (upper ? a[e] : bq[e]) * fast_exp2(upper ? p8[e] : s8[e]);
-                    D8 X = pack8<T>(x);
-                    Gl[L_] = mma_d(X, X, Gl[L_]);
-                    hier_step<h_>(p8, s8, upper);
-                };
-                level(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
-                level(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
-                level(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
-                level(std::integral_constant<int, 8>{}, std::integral_constant<int, 3>{});
-                // p8 = l_i, s8 = tau - l_i.  Rescaled operands, diagonal, table of exp(tau).
-                if (r == 0) {
-                    f32x8 t;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p8[e] + s8[e]);
-                    st8(rtab + w * D + 32 * ks + 8 * c, t);
-                }
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    dot += a[e] * bq[e];
-                    qh[8 * ks + e] = a[e] * fast_exp2(p8[e]);
-                    bq[e] *= fast_exp2(s8[e]);
-                }
-                if (w < NB - 1) st8(Kh + wrow + 32 * ks, pack8<T>(bq));
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            dot = reduce_over_cgroups(dot);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int j = 4 * c + e;
-                float acc = (j == r) ? dot : 0.f;                  // plain fp32 dot on the diagonal (gla.py:983)
-#pragma unroll
-                for (int l = 0; l < 4; ++l) {
-                    const int h_ = 1 << l;
-                    const bool ok = ((j ^ r) < 2 * h_) && (r & h_) && !(j & h_);
-                    acc += ok ? Gl[l][e] : 0.f;
-                }
-                accD[e] = acc;
-            }
-        }
+        subblock_forward<T, D>(p, qf, kf, g + rowoff, q + rowoff, k + rowoff, true, rtab + w * D, Kh + wrow,
+                               w < NB - 1, nullptr, r, c, accD, qh);
     }
     // Values and the first state rows are requested only now: the registers above are free again, and
     // the other workgroup on the CU covers the wait.
