@@ -187,8 +187,12 @@ def bench_recurrent(B, T, H, D, shift, steps, warmup):
     ms_f = time_events(fwd, max(steps, 5), 2)
     ms_b = time_events(bwd, max(steps, 5), 2)
     alg = 34 * D * n_th
-    per = {"recurrent_fwd_kernel": {"ms": round(ms_f, 5), "alg_GBs": round(12 * D * n_th / ms_f / 1e6, 1)},
-           "recurrent_bwd (2 sweeps)": {"ms": round(ms_b, 5), "alg_GBs": round(22 * D * n_th / ms_b / 1e6, 1)}}
+    # (the backward really moves 38*D bytes per token-head: both sweeps read g, q, k, v, dout and q*dq
+    # makes an fp32 round trip, as in the reference's two-sweep kernel)
+    per = {"recurrent_stream_fwd_kernel": {"ms": round(ms_f, 5), "alg_GBs": round(12 * D * n_th / ms_f / 1e6, 1)},
+           "recurrent_stream_dq_kernel + recurrent_stream_rev_kernel": {
+               "ms": round(ms_b, 5), "alg_GBs": round(22 * D * n_th / ms_b / 1e6, 1),
+               "moved_GBs": round(38 * D * n_th / ms_b / 1e6, 1)}}
     achieved = alg / ms_step / 1e6
     return {
         "value": B * T / ms_step / 1e3,
