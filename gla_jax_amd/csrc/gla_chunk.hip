@@ -10,6 +10,7 @@ namespace gla {
 struct ChunkPlan {
     int C = 0;       // tokens per workgroup actually used (a divisor of chunk_size)
     size_t prod = 0, decay = 0, states = 0;   // byte sizes, each rounded up to 256
+    size_t resid = 0;                         // the forward residual: N + 1 states per (b,h), the last one final
 };
 
 static size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -39,6 +40,7 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
     plan->prod = round256((size_t)B * H * N * DK * DV * sizeof(float));
     plan->decay = round256((size_t)B * H * N * DK * sizeof(float));
     plan->states = round256((size_t)B * H * N * DK * DV * esz);
+    plan->resid = round256((size_t)B * H * (N + 1) * DK * DV * esz);
     return GLA_OK;
 }
 
@@ -60,7 +62,7 @@ extern "C" size_t gla_chunk_states_bytes(int64_t B, int64_t T, int64_t H, int64_
                                          int64_t chunk_size, gla_dtype dtype)
 {
     ChunkPlan p;
-    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.states : 0;
+    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.resid : 0;
 }
 
 extern "C" size_t gla_chunk_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
@@ -110,7 +112,7 @@ extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t
         if (e) return e;
         if (stages & 2)
             e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 0, hidden_init, prodT, decay, statesT, states,
-                                         hidden_final);
+                                         hidden_final, 1);
         if (e) return e;
         if (stages & 4)
             e = launch_chunk_out<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, statesT, out);
@@ -162,11 +164,11 @@ extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t
         if (e) return e;
         if (stages & 2)
             e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 1, dhidden_final, prodT, decay, dstatesT, dstatesN,
-                                         dhidden_init);
+                                         dhidden_init, 0);
         if (e) return e;
         if (stages & 4)
             e = launch_chunk_grad<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,
-                                             states, dstatesT, dstatesN, decay, dlog_fgate, dvalue, dkey, dquery);
+                                             states, dstatesT, dstatesN, dlog_fgate, dvalue, dkey, dquery);
         return e;
     });
 }

@@ -37,8 +37,7 @@ template <typename T, int C, int D>
 __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k,
     const T *__restrict__ q, const T *__restrict__ dout, const T *__restrict__ statesN,
-    const T *__restrict__ dstatesT, const T *__restrict__ dstatesN, const float *__restrict__ decay,
-    float *__restrict__ dg, T *__restrict__ dv, T *__restrict__ dk, T *__restrict__ dq, int T_len, int H)
+    const T *__restrict__ dstatesT, const T *__restrict__ dstatesN, float *__restrict__ dg, T *__restrict__ dv, T *__restrict__ dk, T *__restrict__ dq, int T_len, int H)
 {
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4;
     constexpr int LS = TileGeom<T, D>::kStride;
@@ -78,17 +77,20 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     T *sS = tV, *sDn = tV + 32 * LS, *sDt = tV + 64 * LS;
     constexpr int kPieces = 32 * D / 8;                       // 8-element pieces of one staged operand
     constexpr int kPer = (kPieces + C * 4 - 1) / (C * 4);     // pieces per thread
-    D8 pfS[kPer], pfDn[kPer], pfDt[kPer];
+    D8 pfS[kPer], pfS1[kPer], pfDn[kPer], pfDt[kPer];
     f32x8 gN;                                                 // per-row inputs of the next slice
     D8 qN, kN;
     auto stage_fetch = [&](int slice) {
-        const T *Sn = statesN + bhn * D * D, *dSn = dstatesN + bhn * D * D, *dSt = dstatesT + bhn * D * D;
+        // the residual holds N + 1 states per (b,h): slot n is the state before chunk n, slot N the final one
+        const T *Sn = statesN + (bhn + ((int64_t)b * H + h)) * D * D;
+        const T *dSn = dstatesN + bhn * D * D, *dSt = dstatesT + bhn * D * D;
 #pragma unroll
         for (int u = 0; u < kPer; ++u) {
             const int idx = threadIdx.x + u * C * 4;
             if (kPieces % (C * 4) == 0 || idx < kPieces) {
                 const int off = (32 * slice + idx / (D / 8)) * D + (idx % (D / 8)) * 8;
                 pfS[u] = ld8(Sn + off);
+                pfS1[u] = ld8(Sn + D * D + off);
                 pfDn[u] = ld8(dSn + off);
                 pfDt[u] = ld8(dSt + off);
             }
@@ -108,10 +110,11 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 st8(sS + row * LS + c8, pfS[u]);
                 st8(sDn + row * LS + c8, pfDn[u]);
                 st8(sDt + row * LS + c8, pfDt[u]);
-                // chunk-level gate gradient, state part: e^{L_end} * sum_v S_n * dS'  (gla.py:782); the
-                // D/8 threads that hold one row are neighbours in a wave
+                // chunk-level gate gradient (gla.py:782): both of its terms scale with e^{L_end}, like the state
+                // after the chunk, so it equals sum_v dS' * S_{n+1}.  The D/8 threads that hold one row are
+                // neighbours in a wave.
                 float x[8], y[8], part = 0.f;
-                unpack8(pfS[u], x);
+                unpack8(pfS1[u], x);
                 unpack8(pfDn[u], y);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) part += x[e] * y[e];
@@ -119,7 +122,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 part += dpp_f32<kDppQuadXor2>(part);
                 part += dpp_f32<kDppRowHalfMirror>(part);
                 if constexpr (D / 8 == 16) part += dpp_f32<kDppRowMirror>(part);
-                if (c8 == 0) atomicAdd(lbar + 32 * slice + row, part * decay[bhn * D + 32 * slice + row]);
+                if (c8 == 0) lbar[32 * slice + row] = part;
             }
         }
     };
@@ -153,7 +156,6 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             dof[ks] = ld8(dout + rowoff + 32 * ks + 8 * c);
         }
         stage_fetch(0);
-        if (threadIdx.x < D) lbar[threadIdx.x] = 0.f;
 
         // dAn[e] = dA[i = 4c+e][j = r],  dAt[e] = dA[i = r][j = 4c+e]   (dA = dO V^T), own sub-block
         f32x4 dAn = {0.f, 0.f, 0.f, 0.f}, dAt = {0.f, 0.f, 0.f, 0.f};
@@ -471,23 +473,6 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             }
             float kr[8];
             unpack8(ld8(tK + wrow + fo), kr);              // k e^{tau-l} as the MFMAs saw it
-            // chunk-level gate gradient, key part: sum_j (k e^{L_end - L_j}) * (V dS'^T)_j, with
-            // k e^{L_end - L_j} = (k e^{tau - l_j}) * prod_{m > w} r_m
-            {
-                float sig[8];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) sig[e] = 1.f;
-                for (int m = w + 1; m < NB; ++m) {
-                    f32x8 rr = ld8(rtab + m * D + fo + 8 * c);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) sig[e] *= rr.v[e];
-                }
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    float z = reduce_over_rows(kr[e] * acc[e >> 2][e & 3]) * sig[e];
-                    if (r == 0) atomicAdd(lbar + fo + 8 * c + e, z);
-                }
-            }
 #pragma unroll
             for (int I = NB - 1; I >= 1; --I) {
                 if (I > w) {
@@ -560,7 +545,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
 template <typename T, int C, int D>
 int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
                       const void *q, const void *dout, const void *statesN, const void *dstatesT,
-                      const void *dstatesN, const float *decay, float *dg, void *dv, void *dk, void *dq)
+                      const void *dstatesN, float *dg, void *dv, void *dk, void *dq)
 {
     constexpr int LS = TileGeom<T, D>::kStride;
     constexpr int XS = 32 + 16 / (int)sizeof(T);
@@ -572,16 +557,14 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
     if (int e = allow_lds((const void *)kern, lds)) return e;
     dim3 grid(T_len / C * H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
-                       (const T *)dout, (const T *)statesN, (const T *)dstatesT, (const T *)dstatesN, decay,
-                       dg, (T *)dv, (T *)dk, (T *)dq, T_len, H);
+                       (const T *)dout, (const T *)statesN, (const T *)dstatesT, (const T *)dstatesN, dg, (T *)dv, (T *)dk, (T *)dq, T_len, H);
     return launch_status();
 }
 
 #define GLA_INST_GRAD(T, C, D)                                                                           \
     template int launch_chunk_grad<T, C, D>(hipStream_t, int, int, int, const float *, const void *,     \
                                             const void *, const void *, const void *, const void *,     \
-                                            const void *, const void *, const float *, float *, void *,  \
-                                            void *, void *);
+                                            const void *, const void *, float *, void *, void *, void *);
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_GRAD)
 
 }  // namespace gla

@@ -22,7 +22,7 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
 
 template <typename T, int D>
 int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hin, const float *prodT,
-                      const float *decay, void *statesT, void *statesN, void *hout);
+                      const float *decay, void *statesT, void *statesN, void *hout, int tail);
 
 template <typename T, int C, int D>
 int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
@@ -31,6 +31,6 @@ int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, co
 template <typename T, int C, int D>
 int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
                       const void *q, const void *dout, const void *statesN, const void *dstatesT,
-                      const void *dstatesN, const float *decay, float *dg, void *dv, void *dk, void *dq);
+                      const void *dstatesN, float *dg, void *dv, void *dk, void *dq);
 
 }  // namespace gla

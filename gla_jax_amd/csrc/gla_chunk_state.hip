@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ h
                                                          const float *__restrict__ prodT,
                                                          const float *__restrict__ decay,
                                                          T *__restrict__ statesT, T *__restrict__ statesN,
-                                                         T *__restrict__ hout, int N, int reverse)
+                                                         T *__restrict__ hout, int N, int reverse, int tail)
 {
     typedef typename Pair<T>::type P2;
     constexpr int TPD = D / 32;
@@ -164,6 +164,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ h
     const float *pp = prodT + (int64_t)bh * N * D * D + dv0 * D + dk0;
     const float *dp = decay + (int64_t)bh * N * D + dk0;
     const int64_t sbase = (int64_t)bh * N * D * D;
+    const int64_t sbaseN = (int64_t)bh * (N + tail) * D * D;   // tail: one more slot holds the state after the last chunk
     auto emit = [&](int n) {
         if (statesT) {
 #pragma unroll
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ h
             for (int j = 0; j < 2; ++j) {
                 P2 t;
                 t[0] = X[0][j]; t[1] = X[1][j];
-                *reinterpret_cast<P2 *>(statesN + sbase + (int64_t)n * D * D + (dk0 + j) * D + dv0) = t;
+                *reinterpret_cast<P2 *>(statesN + sbaseN + (int64_t)n * D * D + (dk0 + j) * D + dv0) = t;
             }
         }
     };
@@ -215,6 +216,14 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ h
             X[1][j] = dc[j] * X[1][j] + p1[j];
         }
     }
+    if (tail && statesN) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            P2 t;
+            t[0] = X[0][j]; t[1] = X[1][j];
+            *reinterpret_cast<P2 *>(statesN + sbaseN + (int64_t)N * D * D + (dk0 + j) * D + dv0) = t;
+        }
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         P2 t;
@@ -244,11 +253,11 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
 
 template <typename T, int D>
 int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hin, const float *prodT,
-                      const float *decay, void *statesT, void *statesN, void *hout)
+                      const float *decay, void *statesT, void *statesN, void *hout, int tail)
 {
     dim3 grid((D / 32) * (D / 32), BH), block(256);
     hipLaunchKernelGGL((chunk_scan_kernel<T, D>), grid, block, 0, st, (const T *)hin, prodT, decay,
-                       (T *)statesT, (T *)statesN, (T *)hout, N, reverse);
+                       (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
     return launch_status();
 }
 
@@ -257,7 +266,7 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hi
                                              const void *, float *, float *);
 #define GLA_INST_SCAN(T, D)                                                                           \
     template int launch_chunk_scan<T, D>(hipStream_t, int, int, int, const void *, const float *,     \
-                                         const float *, void *, void *, void *);
+                                         const float *, void *, void *, void *, int);
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUTER)
 GLA_INST_SCAN(__bf16, 64)
 GLA_INST_SCAN(__bf16, 128)

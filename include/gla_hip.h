@@ -101,7 +101,8 @@ int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK,
 /* ---- chunk_gla (gla.py:657-692) -------------------------------------------------------------- */
 
 /* Bytes of the `states` residual written by gla_chunk_fwd and read by gla_chunk_bwd: the
- * chunk-start states [B,H,T/C,DK,DV], the analogue of the reference's saved `state` (gla.py:548, 729).
+ * states before every chunk and after the last one, [B,H,T/C+1,DK,DV] in the element type, the analogue of
+ * the reference's saved `state` (gla.py:548, 729; its last slice is hidden_final, gla.py:720-723).
  * Returns 0 for unsupported arguments. */
 size_t gla_chunk_states_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
                               int64_t chunk_size, gla_dtype dtype);
