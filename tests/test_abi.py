@@ -41,9 +41,9 @@ def test_chunk_plan_and_sizes():
     B, T, H, D = 4, 4096, 6, 128
     n_chunks = T // 128
     st = lib.gla_chunk_states_bytes(B, T, H, D, D, 128, _lib.GLA_BF16)
-    assert st == B * H * n_chunks * D * D * 2
+    assert st == B * H * (n_chunks + 1) * D * D * 2      # states before every chunk + the final one
     ws = lib.gla_chunk_fwd_workspace_bytes(B, T, H, D, D, 128, _lib.GLA_BF16)
-    assert ws >= B * H * n_chunks * (D * D * 4 + D * 4) + st
+    assert ws >= B * H * n_chunks * (D * D * 4 + D * 4 + D * D * 2)
     # chunk sizes above the largest tile reuse it; unsupported combinations report 0
     assert lib.gla_chunk_states_bytes(B, T, H, D, D, 256, _lib.GLA_BF16) == st
     assert lib.gla_chunk_states_bytes(B, T, H, D, D, 96, _lib.GLA_BF16) == 0      # not a power of two
