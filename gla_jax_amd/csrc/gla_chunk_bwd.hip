@@ -37,7 +37,8 @@ template <typename T, int C, int D>
 __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k,
     const T *__restrict__ q, const T *__restrict__ dout, const T *__restrict__ statesN,
-    const T *__restrict__ dstatesT, const T *__restrict__ dstatesN, float *__restrict__ dg, T *__restrict__ dv, T *__restrict__ dk, T *__restrict__ dq, int T_len, int H)
+    const T *__restrict__ dstatesT, const T *__restrict__ dstatesN, float *__restrict__ dg,
+    T *__restrict__ dv, T *__restrict__ dk, T *__restrict__ dq, int T_len, int H)
 {
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4;
     constexpr int LS = TileGeom<T, D>::kStride;
@@ -557,7 +558,8 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
     if (int e = allow_lds((const void *)kern, lds)) return e;
     dim3 grid(T_len / C * H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
-                       (const T *)dout, (const T *)statesN, (const T *)dstatesT, (const T *)dstatesN, dg, (T *)dv, (T *)dk, (T *)dq, T_len, H);
+                       (const T *)dout, (const T *)statesN, (const T *)dstatesT, (const T *)dstatesN, dg,
+                       (T *)dv, (T *)dk, (T *)dq, T_len, H);
     return launch_status();
 }
 

@@ -174,7 +174,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
         }
 
         // ---- out^T[dv][i] in slices of 32 output features: state term, then the score blocks --------
-#pragma unroll 1
+#pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const int fo = 32 * ks;
             f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
