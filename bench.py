@@ -35,7 +35,7 @@ FP32_VALU_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (scaled by what the same counters read for a 256 MiB device copy); the runs and their figures
 # are summarised under profiles/.  Keyed by (kernel, B, T, H, D, chunk); absent = not measured.
-MEASURED_TRAFFIC = {("chunk_grad_kernel", 4, 4096, 6, 128, 128): 466.3e6}
+MEASURED_TRAFFIC = {("chunk_grad_kernel", 4, 4096, 6, 128, 128): 496.5e6}
 
 WORKLOADS = {
     # name: (kind, B, T, H, D, chunk, gate shift)
