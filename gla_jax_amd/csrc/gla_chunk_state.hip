@@ -139,7 +139,9 @@ template <typename T> struct Pair;
 template <> struct Pair<__bf16> { typedef bf16x2 type; };
 template <> struct Pair<float> { typedef f32x2 type; };
 
-template <typename T, int D>
+// U = chunks whose inputs are in flight per thread: 4 when the grid fills the machine, 16 when few (b,h)
+// pairs leave it to the single thread to keep the memory system busy (long sequences, small batch).
+template <typename T, int D, int U>
 __global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ hin,
                                                          const float *__restrict__ prodT,
                                                          const float *__restrict__ decay,
@@ -183,7 +185,6 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ h
             }
         }
     };
-    constexpr int U = 4;
     int step = 0;
     for (; step + U <= N; step += U) {
         f32x2 pv[U][2], dc[U];
@@ -256,8 +257,12 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hi
                       const float *decay, void *statesT, void *statesN, void *hout, int tail)
 {
     dim3 grid((D / 32) * (D / 32), BH), block(256);
-    hipLaunchKernelGGL((chunk_scan_kernel<T, D>), grid, block, 0, st, (const T *)hin, prodT, decay,
-                       (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
+    if ((int64_t)grid.x * BH >= 256)
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 4>), grid, block, 0, st, (const T *)hin, prodT, decay,
+                           (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
+    else
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 16>), grid, block, 0, st, (const T *)hin, prodT, decay,
+                           (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
     return launch_status();
 }
 
