@@ -134,12 +134,6 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
 
         // ---- earlier sub-blocks J < w, walking the q side down; scores kept as packed MFMA operands ----
         // (operands and scores as bf16 head + remainder: the products keep 16 bits of mantissa)
-        auto split4 = [](f32x4 x, T4 &hi, T4 &lo) {
-            hi = pack4<T>(x);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) x[e] -= (float)hi[e];
-            lo = pack4<T>(x);
-        };
         T4 sc[NB], sl[NB];
 #pragma unroll
         for (int J = NB - 2; J >= 0; --J) {
@@ -156,12 +150,12 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
                     for (int e = 0; e < 8; ++e) qh[8 * ks + e] *= rr.v[e];
                 }
             }
-            split4(a, sc[J], sl[J]);
+            split4<T>(a, sc[J], sl[J]);
         }
         sc[NB - 1] = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
         sl[NB - 1] = sc[NB - 1];
         T4 scD, slD;
-        split4(accD, scD, slD);
+        split4<T>(accD, scD, slD);
         D8 qb[KS], ql[KS];                   // q * exp(L_i), operand of the state term: bf16 head and remainder
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
