@@ -42,6 +42,8 @@ WORKLOADS = {
     "chunk": ("chunk", 4, 4096, 6, 128, 128, 5.0),       # BASELINE configs[1]/[2] (headline metric)
     "long": ("chunk", 1, 32768, 8, 128, 128, 0.0),       # BASELINE configs[3]
     "recurrent": ("recurrent", 16, 2048, 16, 64, 0, 3.0),  # BASELINE configs[4]
+    # the two scan operators of ops.py on their own, at the sizes chunk_gla gives them at the headline shape
+    "scans": ("scans", 4, 4096, 6, 128, 128, 5.0),
 }
 
 
@@ -206,6 +208,56 @@ def bench_recurrent(B, T, H, D, shift, steps, warmup):
     }
 
 
+def bench_scans(B, T, H, D, chunk, shift, steps, warmup):
+    """cumsum_recursive of the gates along T ([B,T,H,D] fp32) and rnn_recursive over the chunks
+    ([B*H, T/chunk, D] gates, [B*H, T/chunk, D, D] products, fp32): 8 bytes per element each."""
+    import torch
+    from gla_jax_amd import _lib
+    lib = _lib.load()
+    g = torch.nn.functional.logsigmoid(shift + torch.randn(B, T, H, D, device="cuda")).contiguous()
+    dst = torch.empty_like(g)
+    N = T // chunk
+    a = torch.nn.functional.logsigmoid(torch.randn(B * H, N, D, device="cuda")).contiguous()
+    kv = torch.randn(B * H, N, D, D, device="cuda")
+    oa, ob = torch.empty_like(a), torch.empty_like(kv)
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda t: t.data_ptr()
+
+    def cum():
+        _lib.check("gla_cumsum_f32", lib.gla_cumsum_f32(st, p(g), None, p(dst), B, T, H * D, 0))
+
+    def rnn():
+        _lib.check("gla_rnn_scan_f32", lib.gla_rnn_scan_f32(st, p(a), p(kv), None, None, p(oa), p(ob), B * H, N, D,
+                                                          D, 0))
+
+    def step():
+        cum()
+        rnn()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+    ms_c = time_events(cum, max(steps, 10), 3)
+    ms_r = time_events(rnn, max(steps, 10), 3)
+    bc, br = 8 * g.numel(), 8 * kv.numel() + 8 * a.numel()
+    per = {"cumsum_kernel": {"ms": round(ms_c, 5), "alg_GBs": round(bc / ms_c / 1e6, 1)},
+           "rnn_scan_kernel": {"ms": round(ms_r, 5), "alg_GBs": round(br / ms_r / 1e6, 1)}}
+    dom, dom_b, dom_ms = ("rnn_scan_kernel", br, ms_r) if ms_r > ms_c else ("cumsum_kernel", bc, ms_c)
+    return {
+        "value": (bc + br) / ms_step / 1e6,
+        "ms_per_step": ms_step,
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(dom_b / dom_ms / 1e6, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_b / dom_ms / 1e6 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "alg_bytes_per_launch": dom_b},
+        "kernels": per,
+    }
+
+
 def cpu_baseline(B, T, H, D, shift, budget_s=12.0):
     """The C restatement of recurrent_gla_naive (oracle/), forward + gradients, on one batch element
     of the workload, repeated until ~budget_s of wall time is spent."""
@@ -259,18 +311,25 @@ def main():
         metric = "chunk_gla fwd+bwd Mtokens/s (B4,T4096,H6,D128 bf16); % bf16 MFMA peak" \
             if args.workload == "chunk" else f"chunk_gla fwd+bwd Mtokens/s (B{B},T{T},H{H},D{D} bf16)"
         wl = f"chunk_gla fwd+bwd B{B} T{T} H{H} D{D} chunk{chunk} bf16, gates log_sigmoid({shift:g}+N(0,1)) fp32"
+    elif kind == "scans":
+        r = bench_scans(B, T, H, D, chunk, shift, args.steps, args.warmup)
+        metric = "ops.py scans (cumsum_recursive + rnn_recursive) GB/s"
+        wl = f"cumsum over T of [B{B},T{T},H{H},D{D}] fp32 + diagonal RNN scan over {T // chunk} chunks of [{B * H},{D},{D}] fp32"
     else:
         r = bench_recurrent(B, T, H, D, shift, args.steps, args.warmup)
         metric = f"recurrent_gla fwd+bwd Mtokens/s (B{B},T{T},H{H},D{D} bf16); HBM GB/s"
         wl = f"recurrent_gla fwd+bwd B{B} T{T} H{H} D{D} bf16, gates log_sigmoid({shift:g}+N(0,1)) fp32"
     line = {
-        "metric": metric, "value": round(r.pop("value"), 4), "unit": "Mtokens/s", "n_gpus": 1,
+        "metric": metric, "value": round(r.pop("value"), 4), "unit": "GB/s" if kind == "scans" else "Mtokens/s",
+        "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(r.pop("ms_per_step"), 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic", "config": {"workload": wl, "B": B, "T": T, "H": H, "D": D, "chunk_size": chunk},
     }
     line.update(r)
-    if not args.no_cpu:
+    if kind == "scans":
+        line["dtype"] = "f32"
+    elif not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(B, T, H, D, shift)
     print(json.dumps(line))
 

@@ -72,6 +72,62 @@ __global__ __launch_bounds__(WAVES * 64) void cumsum_kernel(const float *__restr
     }
 }
 
+// The same with the scanned axis cut finer, for long axes over few columns: a block owns CL columns of one
+// outer index, a wave covers 64 / CL segments at once (lane = segment-in-wave x column), the block
+// WAVES * 64 / CL segments.  A wave access is 64 / CL row pieces of CL floats.
+template <int CL, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void cumsum_tiled_kernel(const float *__restrict__ src,
+                                                                  const float *__restrict__ init,
+                                                                  float *__restrict__ dst, int64_t t_len,
+                                                                  int64_t n_inner, int reverse)
+{
+    constexpr int TG = 64 / CL, NSEG = WAVES * TG;
+    __shared__ float totals[NSEG][CL];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int cl = lane % CL, segi = wave * TG + lane / CL;
+    const int64_t col = (int64_t)blockIdx.x * CL + cl;
+    const int64_t outer = blockIdx.y;
+    const bool valid = col < n_inner;
+    const int64_t seg = (t_len + NSEG - 1) / NSEG;
+    const int64_t s0 = segi * seg < t_len ? segi * seg : t_len;
+    const int64_t s1 = s0 + seg < t_len ? s0 + seg : t_len;
+    const float *base = src + outer * t_len * n_inner + col;
+    float *obase = dst + outer * t_len * n_inner + col;
+
+    float sum = 0.f;
+    if (valid) {
+        int64_t s = s0;
+        for (; s + 8 <= s1; s += 8) {
+            float a[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) a[u] = base[(reverse ? t_len - 1 - (s + u) : s + u) * n_inner];
+            sum += ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
+        }
+        for (; s < s1; ++s) sum += base[(reverse ? t_len - 1 - s : s) * n_inner];
+    }
+    totals[segi][cl] = sum;
+    __syncthreads();
+    if (!valid) return;
+    float run = init ? init[outer * n_inner + col] : 0.f;
+    for (int w = 0; w < segi; ++w) run += totals[w][cl];
+    int64_t s = s0;
+    for (; s + 8 <= s1; s += 8) {
+        float a[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a[u] = base[(reverse ? t_len - 1 - (s + u) : s + u) * n_inner];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            run += a[u];
+            obase[(reverse ? t_len - 1 - (s + u) : s + u) * n_inner] = run;
+        }
+    }
+    for (; s < s1; ++s) {
+        const int64_t t = reverse ? t_len - 1 - s : s;
+        run += base[t * n_inner];
+        obase[t * n_inner] = run;
+    }
+}
+
 // One thread = one (k, 4 consecutive v) strip of the state, walked over T in registers; the loads
 // of step n do not depend on the recurrence, so UNROLL of them are kept in flight.
 template <int UNROLL>
@@ -134,7 +190,12 @@ extern "C" int gla_cumsum_f32(void *stream, const float *src, const float *init,
     if (n_outer <= 0 || t_len <= 0 || n_inner <= 0 || n_outer > 65535) return GLA_ERR_SHAPE;
     dim3 grid((unsigned)((n_inner + 63) / 64), (unsigned)n_outer);
     hipStream_t st = (hipStream_t)stream;
-    if (t_len >= 64)
+    // long axis over few columns: cut the axis finer so that the grid fills the machine
+    if (t_len >= 2048 && (int64_t)grid.x * grid.y < 1024) {
+        dim3 fine((unsigned)((n_inner + 15) / 16), (unsigned)n_outer);
+        hipLaunchKernelGGL((gla::cumsum_tiled_kernel<16, 16>), fine, dim3(1024), 0, st, src, init, dst, t_len,
+                           n_inner, reverse);
+    } else if (t_len >= 64)
         hipLaunchKernelGGL(gla::cumsum_kernel<4>, grid, dim3(256), 0, st, src, init, dst, t_len, n_inner,
                            reverse);
     else
