@@ -26,7 +26,8 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
     if (DK != DV) return GLA_ERR_SHAPE;                      // gla.py:499
     if (!is_pow2(chunk) || T % chunk != 0) return GLA_ERR_CHUNK;   // gla.py:500, 674
     int64_t C = chunk;
-    const int64_t cmax = dtype == GLA_BF16 ? 128 : 64;
+    // largest tile built: 128 tokens for bf16, for fp32 (tiles twice as wide) 64 at D=64 and 32 at D=128
+    const int64_t cmax = dtype == GLA_BF16 ? 128 : (DK > 64 ? 32 : 64);
     if (C > cmax) C = cmax;
     bool ok = false;
 #define GLA_PLAN_CASE(T_, C_, D_) \

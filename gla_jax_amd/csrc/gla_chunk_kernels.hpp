@@ -10,11 +10,13 @@ namespace gla {
 #define GLA_FOR_EACH_CHUNK_CONFIG(M) \
     M(__bf16, 128, 128)              \
     M(__bf16, 64, 128)               \
+    M(__bf16, 32, 128)               \
     M(__bf16, 128, 64)               \
     M(__bf16, 64, 64)                \
     M(__bf16, 32, 64)                \
     M(float, 64, 64)                 \
-    M(float, 32, 64)
+    M(float, 32, 64)                 \
+    M(float, 32, 128)
 
 template <typename T, int C, int D>
 int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const float *g, const void *x,

@@ -49,7 +49,9 @@ def test_chunk_plan_and_sizes():
     assert lib.gla_chunk_states_bytes(B, T, H, D, D, 96, _lib.GLA_BF16) == 0      # not a power of two
     assert lib.gla_chunk_states_bytes(B, 100, H, D, D, 64, _lib.GLA_BF16) == 0    # does not divide T
     assert lib.gla_chunk_states_bytes(B, T, H, 128, 64, 128, _lib.GLA_BF16) == 0  # DK != DV
-    assert lib.gla_chunk_states_bytes(B, T, H, D, D, 128, _lib.GLA_F32) == 0      # fp32 is built for D=64
+    # fp32 at D=128 runs on the 32-token tile: 4x as many chunks, 4-byte elements
+    assert lib.gla_chunk_states_bytes(B, T, H, D, D, 128, _lib.GLA_F32) == B * H * (4 * n_chunks + 1) * D * D * 4
+    assert lib.gla_chunk_states_bytes(B, T, H, 256, 256, 128, _lib.GLA_BF16) == 0  # head dims built: 64, 128
 
 
 def test_entry_points_reject_bad_arguments_without_touching_the_gpu():

@@ -21,6 +21,8 @@ CASES = [
     (torch.bfloat16, 1, 512, 1, 128, 256, 5.0),     # chunk above the largest tile: same result
     (torch.float32, 1, 512, 2, 64, 64, 5.0),        # BASELINE configs[0]
     (torch.float32, 2, 128, 1, 64, 32, 0.0),
+    (torch.bfloat16, 1, 256, 2, 128, 32, 2.0),      # the smallest tile at D=128
+    (torch.float32, 1, 256, 2, 128, 128, 4.0),      # fp32 at D=128 runs on the 32-token tile
 ]
 
 
