@@ -90,10 +90,10 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             const int idx = threadIdx.x + u * C * 4;
             if (kPieces % (C * 4) == 0 || idx < kPieces) {
                 const int off = (32 * slice + idx / (D / 8)) * D + (idx % (D / 8)) * 8;
-                pfS[u] = ld8(Sn + off);
-                pfS1[u] = ld8(Sn + D * D + off);
-                pfDn[u] = ld8(dSn + off);
-                pfDt[u] = ld8(dSt + off);
+                pfS[u] = ld8_once(Sn + off);
+                pfS1[u] = ld8_once(Sn + D * D + off);
+                pfDn[u] = ld8_once(dSn + off);
+                pfDt[u] = ld8_once(dSt + off);
             }
         }
     };
@@ -153,8 +153,8 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
         }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            vf[ks] = ld8(v + rowoff + 32 * ks + 8 * c);
-            dof[ks] = ld8(dout + rowoff + 32 * ks + 8 * c);
+            vf[ks] = ld8_once(v + rowoff + 32 * ks + 8 * c);
+            dof[ks] = ld8_once(dout + rowoff + 32 * ks + 8 * c);
         }
         stage_fetch(0);
 
@@ -461,7 +461,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 o[e] = fast_exp2(p8[e]) * hacc + dq8[e];
                 dl8[e] += qr[e] * hacc;
             }
-            st8(dq + rowoff + fo + 8 * c, pack8<T>(o));
+            st8_once(dq + rowoff + fo + 8 * c, pack8<T>(o));
         }
         // -- dk: state term V dS'^T first, then the later sub-blocks in descending order
         {
@@ -493,7 +493,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 o[e] = fast_exp2(s8[e]) * hacc + dk8[e];
                 dl8[e] -= kr[e] * hacc;
             }
-            st8(dk + rowoff + fo + 8 * c, pack8<T>(o));
+            st8_once(dk + rowoff + fo + 8 * c, pack8<T>(o));
         }
         // -- dv: state term K~ dS' first, then the own and the later sub-blocks
         {
@@ -516,7 +516,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             float o[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
-            st8(dv + rowoff + fo + 8 * c, pack8<T>(o));
+            st8_once(dv + rowoff + fo + 8 * c, pack8<T>(o));
         }
         // -- dL of the slice is complete: reverse cumsum inside the sub-block (gla.py:616-617), then, once
         // every wave has published its sub-block total, over the whole chunk + the chunk-level term (gla.py:782)
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
 #pragma unroll
                 for (int e = 0; e < 8; ++e) o.v[e] += t.v[e];
             }
-            st8(dg + rowoff + fo + 8 * c, o);
+            st8_once(dg + rowoff + fo + 8 * c, o);
         }
         if (ks + 1 < KS) {
             stage_store(ks + 1);

@@ -113,6 +113,32 @@ __device__ __forceinline__ void st8(float *p, const f32x8 &v)
     reinterpret_cast<f32x4 *>(p)[1] = b;
 }
 
+// The same for global data that is touched exactly once (streamed state rows, outputs): non-temporal
+// accesses, which leave the L2 lines of the inputs that are read again alone.
+__device__ __forceinline__ bf16x8 ld8_once(const __bf16 *p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const bf16x8 *>(p));
+}
+__device__ __forceinline__ f32x8 ld8_once(const float *p)
+{
+    f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p)),
+          b = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p) + 1);
+    f32x8 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { r.v[e] = a[e]; r.v[4 + e] = b[e]; }
+    return r;
+}
+__device__ __forceinline__ void st8_once(__bf16 *p, bf16x8 v)
+{
+    __builtin_nontemporal_store(v, reinterpret_cast<bf16x8 *>(p));
+}
+__device__ __forceinline__ void st8_once(float *p, const f32x8 &v)
+{
+    f32x4 a = {v.v[0], v.v[1], v.v[2], v.v[3]}, b = {v.v[4], v.v[5], v.v[6], v.v[7]};
+    __builtin_nontemporal_store(a, reinterpret_cast<f32x4 *>(p));
+    __builtin_nontemporal_store(b, reinterpret_cast<f32x4 *>(p) + 1);
+}
+
 // LDS tiles are row-major [rows][D] with a 16-byte pad per row.
 template <typename T, int D> struct TileGeom {
     static constexpr int kStride = D + 16 / (int)sizeof(T);
