@@ -16,7 +16,8 @@ struct ChunkPlan {
 static size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // The result does not depend on the chunk length (only its rounding does), so chunk sizes above the
-// largest compiled tile run with that tile; sizes below 16 tokens are not built.
+// largest compiled tile run with that tile; sizes below 32 tokens are not built (the leaf of the reference
+// needs 32 rows as well, gla.py:975-977).
 static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, int64_t chunk, int dtype,
                       ChunkPlan *plan)
 {

@@ -1,0 +1,76 @@
+"""The HIP path, through the C ABI, against the committed golden vectors (tests/golden/*.npz): chunk_gla at
+every tile size, recurrent_gla in both directions and both element types, and the two stand-alone scans.
+Tolerance as everywhere (north_star): max|err| / RMS <= 2e-2 for bf16, <= 1e-4 for fp32."""
+import numpy as np
+import pytest
+import torch
+
+from tests.test_golden import GRADS, INPUTS, load
+from tests.util import TOL, assert_close, err_over_rms, grad_kinds, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def device_inputs(d, dtype):
+    return [to_dev(d[k], torch.float32 if k == "log_fgate" else dtype) for k in INPUTS]
+
+
+def check(d, tag, dtype, hT, out, grads):
+    tol = TOL[dtype]
+    assert_close("out", to_np(out), d[f"{tag}_out"], tol, stored=dtype)
+    assert_close("hidden_final", to_np(hT), d[f"{tag}_hidden_final"], tol, stored=dtype)
+    for name, got, st in zip(GRADS, grads, grad_kinds(dtype)):
+        assert_close(name, to_np(got), d[f"{tag}_{name}"], tol, stored=st)
+
+
+def fwd_bwd(fn, d, dtype, **kw):
+    dev = [t.requires_grad_(True) for t in device_inputs(d, dtype)]
+    hT, out = fn(*dev, **kw)
+    loss = (hT.float() * to_dev(d["dhidden_final"], torch.float32)).sum() + \
+           (out.float() * to_dev(d["dout"], torch.float32)).sum()
+    return hT, out, torch.autograd.grad(loss, dev)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("chunk", [32, 64])
+def test_chunk_gla_against_golden(dtype, chunk):
+    from gla_jax_amd import chunk_gla
+    d = load("gla_T64_H1_D64.npz")
+    hT, out, grads = fwd_bwd(chunk_gla, d, dtype, chunk_size=chunk)
+    check(d, "fwd", dtype, hT, out, grads)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_recurrent_gla_against_golden(dtype, reverse):
+    from gla_jax_amd import recurrent_gla
+    d = load("gla_T64_H1_D64.npz")
+    hT, out, grads = fwd_bwd(recurrent_gla, d, dtype, reverse=reverse)
+    check(d, "rev" if reverse else "fwd", dtype, hT, out, grads)
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_recurrent_gla_small_head_dim_against_golden(reverse):
+    """Head dim 8 is below what the kernels are built for: the front-end must refuse it, not fall back."""
+    from gla_jax_amd import recurrent_gla
+    d = load("gla_T12_H2_D8.npz")
+    from gla_jax_amd._lib import GlaError
+    with pytest.raises(GlaError):
+        recurrent_gla(*device_inputs(d, torch.float32), reverse=reverse)
+
+
+def test_scans_against_golden():
+    from gla_jax_amd import cumsum_recursive, rnn_recursive
+    d = load("scans.npz")
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+    for reverse in (False, True):
+        for with_init in (False, True):
+            tag = f"{'rev' if reverse else 'fwd'}_{'init' if with_init else 'noinit'}"
+            got = cumsum_recursive(dev(d["cumsum_src"]), 1, init=dev(d["cumsum_init"]) if with_init else None,
+                                   reverse=reverse)
+            assert err_over_rms(to_np(got), d[f"cumsum_{tag}"]) < 1e-5, tag
+            ga, gx = rnn_recursive(dev(d["rnn_log_fgate"]), dev(d["rnn_kv"]),
+                                   dev(d["rnn_init_log_fgate"]) if with_init else None,
+                                   dev(d["rnn_init_kv"]) if with_init else None, reverse=reverse)
+            assert err_over_rms(to_np(ga), d[f"rnn_a_{tag}"]) < 1e-5, tag
+            assert err_over_rms(to_np(gx), d[f"rnn_x_{tag}"]) < 1e-5, tag
