@@ -37,6 +37,7 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
 #undef GLA_PLAN_CASE
     if (!ok) return GLA_ERR_UNSUPPORTED;
     const size_t N = (size_t)(T / C);
+    if ((int64_t)N * H > 0x7fffffffLL) return GLA_ERR_SHAPE;   // chunks x heads is the grid's x extent
     const size_t esz = dtype == GLA_BF16 ? 2 : 4;
     plan->C = (int)C;
     plan->prod = round256((size_t)B * H * N * DK * DV * sizeof(float));

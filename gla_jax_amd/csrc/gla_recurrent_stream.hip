@@ -116,15 +116,21 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
         {
             float p[NV];
             D8 qf[KS], kf[KS];
+            if ((n + 1) * C > T_len && !valid) {   // only the last block can hold padded steps
+                float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    gN[ks] = pack8<float>(z);
+                    qN[ks] = kN[ks] = vN[ks] = pack8<T>(z);
+                }
+            }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                const D8 z8 = pack8<T>(z);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) p[8 * ks + e] = valid ? gN[ks].v[e] * kLog2e : 0.f;
-                qf[ks] = valid ? qN[ks] : z8;
-                kf[ks] = valid ? kN[ks] : z8;
-                st8(Vn + wrow + 32 * ks, valid ? vN[ks] : z8);
+                for (int e = 0; e < 8; ++e) p[8 * ks + e] = gN[ks].v[e] * kLog2e;
+                qf[ks] = qN[ks];
+                kf[ks] = kN[ks];
+                st8(Vn + wrow + 32 * ks, vN[ks]);
             }
             if (n + 1 < N) fetch(n + 1);
             subblock_forward<T, D, true>(p, qf, kf, g + row, q + row, k + row, valid, rtab + w * D, Kh + wrow, true,

@@ -168,16 +168,22 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
         bool one_anchor;
         {
             D8 vf[KS];
-            float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            const D8 z8 = pack8<T>(z);
+            if ((n + 1) * C > T_len && !valid) {   // only the last block can hold padded steps
+                float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    gN[ks] = pack8<float>(z);
+                    qN[ks] = kN[ks] = vN[ks] = dN[ks] = pack8<T>(z);
+                }
+            }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) p[8 * ks + e] = valid ? gN[ks].v[e] * kLog2e : 0.f;
-                qf[ks] = valid ? qN[ks] : z8;
-                kf[ks] = valid ? kN[ks] : z8;
-                vf[ks] = valid ? vN[ks] : z8;
-                dof[ks] = valid ? dN[ks] : z8;
+                for (int e = 0; e < 8; ++e) p[8 * ks + e] = gN[ks].v[e] * kLog2e;
+                qf[ks] = qN[ks];
+                kf[ks] = kN[ks];
+                vf[ks] = vN[ks];
+                dof[ks] = dN[ks];
                 st8(Vn + wrow + 32 * ks, vf[ks]);
             }
             if (n + 1 < N) fetch(n + 1);
@@ -487,19 +493,25 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
         float dd = 0.f;
         {
             float p[NV];
-            float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            const D8 z8 = pack8<T>(z);
+            if ((n + 1) * C > T_len && !valid) {   // only the last block can hold padded steps
+                float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    gN[ks] = wN[ks] = pack8<float>(z);
+                    qN[ks] = kN[ks] = vN[ks] = dN[ks] = pack8<T>(z);
+                }
+            }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    p[8 * ks + e] = valid ? gN[ks].v[e] * kLog2e : 0.f;
-                    qdq[8 * ks + e] = valid ? wN[ks].v[e] : 0.f;
+                    p[8 * ks + e] = gN[ks].v[e] * kLog2e;
+                    qdq[8 * ks + e] = wN[ks].v[e];
                 }
-                qf[ks] = valid ? qN[ks] : z8;
-                kf[ks] = valid ? kN[ks] : z8;
-                vf[ks] = valid ? vN[ks] : z8;
-                dof[ks] = valid ? dN[ks] : z8;
+                qf[ks] = qN[ks];
+                kf[ks] = kN[ks];
+                vf[ks] = vN[ks];
+                dof[ks] = dN[ks];
                 st8(tO + wrow + 32 * ks, dof[ks]);
             }
             if (n > 0) fetch(n - 1);
