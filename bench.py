@@ -35,7 +35,7 @@ FP32_VALU_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (scaled by what the same counters read for a 256 MiB device copy); the runs and their figures
 # are summarised under profiles/.  Keyed by (kernel, B, T, H, D, chunk); absent = not measured.
-MEASURED_TRAFFIC = {("chunk_grad_kernel", 4, 4096, 6, 128, 128): 496.5e6}
+MEASURED_TRAFFIC = {("chunk_grad_kernel", 4, 4096, 6, 128, 128): 428.9e6}
 
 WORKLOADS = {
     # name: (kind, B, T, H, D, chunk, gate shift)
@@ -123,12 +123,12 @@ def bench_chunk(B, T, H, D, chunk, shift, steps, warmup):
         "fwd.chunk_outer_kernel": (lambda: fwd(1), 8 * D * n_th, 8 * D * n_th + state_f32),
         # the scans write the chunk states in both orientations; the gradient kernel reads four state
         # arrays (S_n, S_{n+1}, dS' twice) and the gates, q and k a second time (once for the score
-        # blocks, once per feature slice)
+        # blocks, once per feature slice; about half of that second read is served by the L2: measured)
         "fwd.chunk_scan_kernel": (lambda: fwd(2), 0, state_f32 + 2 * state_bf16),
         "fwd.chunk_out_kernel": (lambda: fwd(4), 12 * D * n_th, 12 * D * n_th + state_bf16),
         "bwd.chunk_outer_kernel": (lambda: bwd(1), 8 * D * n_th, 8 * D * n_th + state_f32),
         "bwd.chunk_scan_kernel": (lambda: bwd(2), 0, state_f32 + 2 * state_bf16),
-        "bwd.chunk_grad_kernel": (lambda: bwd(4), 22 * D * n_th, 30 * D * n_th + 4 * state_bf16),
+        "bwd.chunk_grad_kernel": (lambda: bwd(4), 22 * D * n_th, 26 * D * n_th + 4 * state_bf16),
     }
     per = {}
     for name, (fn, alg, moved) in kernels.items():
