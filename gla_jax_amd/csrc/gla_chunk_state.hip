@@ -139,7 +139,7 @@ template <typename T> struct Pair;
 template <> struct Pair<__bf16> { typedef bf16x2 type; };
 template <> struct Pair<float> { typedef f32x2 type; };
 
-// U = chunks whose inputs are in flight per thread: 4 when the grid fills the machine, 16 when few (b,h)
+// U = chunks whose inputs are in flight per thread: 4 when the grid fills the machine, 32 when few (b,h)
 // pairs leave it to the single thread to keep the memory system busy (long sequences, small batch).
 template <typename T, int D, int U>
 __global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ hin,
@@ -257,12 +257,13 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hi
                       const float *decay, void *statesT, void *statesN, void *hout, int tail)
 {
     dim3 grid((D / 32) * (D / 32), BH), block(256);
-    if ((int64_t)grid.x * BH >= 256)
+    if ((int64_t)grid.x * BH >= 256) {
         hipLaunchKernelGGL((chunk_scan_kernel<T, D, 4>), grid, block, 0, st, (const T *)hin, prodT, decay,
                            (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
-    else
-        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 16>), grid, block, 0, st, (const T *)hin, prodT, decay,
+    } else {
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 32>), grid, block, 0, st, (const T *)hin, prodT, decay,
                            (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
+    }
     return launch_status();
 }
 
