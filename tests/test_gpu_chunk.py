@@ -23,6 +23,8 @@ CASES = [
     (torch.float32, 2, 128, 1, 64, 32, 0.0),
     (torch.bfloat16, 1, 256, 2, 128, 32, 2.0),      # the smallest tile at D=128
     (torch.float32, 1, 256, 2, 128, 128, 4.0),      # fp32 at D=128 runs on the 32-token tile
+    (torch.bfloat16, 3, 128, 5, 128, 128, 3.0),     # a single chunk per sequence, odd batch and head counts
+    (torch.bfloat16, 1, 64, 1, 64, 64, 3.0),
 ]
 
 
