@@ -128,6 +128,47 @@ __global__ __launch_bounds__(WAVES * 64) void cumsum_tiled_kernel(const float *_
     }
 }
 
+// The same for segments of at most SEG rows: a thread keeps its whole segment in registers between the two
+// passes, so the source is read once (all SEG requests go out before the first sum) and nothing is re-read.
+template <int CL, int WAVES, int SEG>
+__global__ __launch_bounds__(WAVES * 64) void cumsum_cached_kernel(const float *__restrict__ src,
+                                                                   const float *__restrict__ init,
+                                                                   float *__restrict__ dst, int64_t t_len,
+                                                                   int64_t n_inner, int reverse)
+{
+    constexpr int TG = 64 / CL, NSEG = WAVES * TG;
+    __shared__ float totals[NSEG][CL];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int cl = lane % CL, segi = wave * TG + lane / CL;
+    const int64_t col = (int64_t)blockIdx.x * CL + cl;
+    const int64_t outer = blockIdx.y;
+    const bool valid = col < n_inner;
+    const int64_t seg = (t_len + NSEG - 1) / NSEG;            // <= SEG, checked by the launcher
+    const int64_t s0 = segi * seg < t_len ? segi * seg : t_len;
+    const int len = valid ? (int)((s0 + seg < t_len ? s0 + seg : t_len) - s0) : 0;
+    // element u of the segment sits `step` rows after the first one (before it when summing from the far end)
+    const int64_t first = reverse ? t_len - 1 - s0 : s0;
+    const int64_t step = reverse ? -n_inner : n_inner;
+    const float *base = src + outer * t_len * n_inner + first * n_inner + (valid ? col : 0);
+    float *obase = dst + outer * t_len * n_inner + first * n_inner + (valid ? col : 0);
+
+    float a[SEG];
+#pragma unroll
+    for (int u = 0; u < SEG; ++u) a[u] = u < len ? base[u * step] : 0.f;
+    float sum = 0.f;
+#pragma unroll
+    for (int u = 0; u < SEG; u += 4) sum += (a[u] + a[u + 1]) + (a[u + 2] + a[u + 3]);
+    totals[segi][cl] = sum;
+    __syncthreads();
+    float run = (init && valid) ? init[outer * n_inner + col] : 0.f;
+    for (int w = 0; w < segi; ++w) run += totals[w][cl];
+#pragma unroll
+    for (int u = 0; u < SEG; ++u) {
+        run += a[u];
+        if (u < len) obase[u * step] = run;
+    }
+}
+
 // One thread = one (k, 4 consecutive v) strip of the state, walked over T in registers; the loads
 // of step n do not depend on the recurrence, so UNROLL of them are kept in flight.
 template <int UNROLL>
@@ -193,9 +234,16 @@ extern "C" int gla_cumsum_f32(void *stream, const float *src, const float *init,
     // long axis over few columns: cut the axis finer so that the grid fills the machine
     if (t_len >= 2048 && (int64_t)grid.x * grid.y < 1024) {
         dim3 fine((unsigned)((n_inner + 15) / 16), (unsigned)n_outer);
-        hipLaunchKernelGGL((gla::cumsum_tiled_kernel<16, 16>), fine, dim3(1024), 0, st, src, init, dst, t_len,
+        if (t_len <= 64 * 64)       // 64 segments of at most 64 rows: held in registers, read once
+            hipLaunchKernelGGL((gla::cumsum_cached_kernel<16, 16, 64>), fine, dim3(1024), 0, st, src, init, dst,
+                               t_len, n_inner, reverse);
+        else
+            hipLaunchKernelGGL((gla::cumsum_tiled_kernel<16, 16>), fine, dim3(1024), 0, st, src, init, dst, t_len,
+                               n_inner, reverse);
+    } else if (t_len >= 64 && t_len <= 4 * 64)
+        hipLaunchKernelGGL((gla::cumsum_cached_kernel<64, 4, 64>), grid, dim3(256), 0, st, src, init, dst, t_len,
                            n_inner, reverse);
-    } else if (t_len >= 64)
+    else if (t_len >= 64)
         hipLaunchKernelGGL(gla::cumsum_kernel<4>, grid, dim3(256), 0, st, src, init, dst, t_len, n_inner,
                            reverse);
     else
