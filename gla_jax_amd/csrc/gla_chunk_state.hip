@@ -33,7 +33,6 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     T *Xn = reinterpret_cast<T *>(smem);
     T *Yn = Xn + C * LS;
     float *rtab = reinterpret_cast<float *>(Yn + C * LS);   // [NB][D] e^{tau_m}
-    float *ttab = rtab + NB * D;                            // [NB][D] tau_m (log2 units)
 
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int r = lane & 15, c = lane >> 4;
@@ -55,19 +54,25 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
         yf[ks] = ld8(y + rowoff + d0);
         xf[ks] = ld8(x + rowoff + d0);
     }
-    // p = gate prefix inside the sub-block (log2 units); row 15 holds the sub-block total tau, which
-    // goes to ttab as it is and to rtab as e^{tau}.
+    // Gate sums inside the sub-block (log2 units).  The query side needs the inclusive prefix l_i, the key
+    // side the sum over the LATER rows, tau - l_j: that one is scanned directly (a suffix scan, then one row
+    // down) instead of being formed as a difference, which would cancel against a closed gate (g = -200
+    // leaves 3e-5 of absolute error in every later prefix).  The row that ends up with the sub-block total
+    // tau (15 for the prefix, 0 for the suffix) publishes e^{tau}.
 #pragma unroll
-    for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
-    if (r == 15) {
+    for (int i = 0; i < NV; ++i) p[i] = MODE == 0 ? suffix_sum_rows(p[i]) : prefix_sum_rows(p[i]);
+    if (r == (MODE == 0 ? 0 : 15)) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             f32x8 t;
 #pragma unroll
             for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p[8 * ks + e]);
-            st8(ttab + w * D + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
             st8(rtab + w * D + 32 * ks + 8 * c, t);
         }
+    }
+    if (MODE == 0) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) p[i] = dpp_f32<0x101>(p[i]);   // row_shl:1: the next row's sum, 0 past the last
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) st8(Xn + (16 * w + r) * LS + 32 * ks + 8 * c, xf[ks]);
@@ -76,14 +81,8 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     for (int ks = 0; ks < KS; ++ks) {
         const int d0 = 32 * ks + 8 * c;
         float f[8], yv[8];
-        if (MODE == 0) {
-            f32x8 tau = ld8(ttab + w * D + d0);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) f[e] = fast_exp2(tau.v[e] - p[8 * ks + e]);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) f[e] = fast_exp2(p[8 * ks + e]);
-        }
+        for (int e = 0; e < 8; ++e) f[e] = fast_exp2(p[8 * ks + e]);
         float all[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) all[e] = 1.f;
@@ -238,7 +237,7 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
                        const void *y, float *prodT, float *decay)
 {
     constexpr int LS = TileGeom<T, D>::kStride;
-    const size_t lds = (size_t)2 * C * LS * sizeof(T) + (size_t)2 * (C / 16) * D * sizeof(float);
+    const size_t lds = (size_t)2 * C * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
     dim3 grid(T_len / C * H, B), block(C * 4);
     if (mode == 0) {
         auto kern = chunk_outer_kernel<T, C, D, 0>;
