@@ -158,8 +158,8 @@ __global__ __launch_bounds__(RK * 64) void recurrent_fwd_kernel(
 template <typename T, typename TO, int RV, int U>
 __global__ __launch_bounds__(RV * 64) void recurrent_bwd_dq_kernel(
     const T *__restrict__ h0, const float *__restrict__ g, const T *__restrict__ v,
-    const T *__restrict__ k, const T *__restrict__ q, const TO *__restrict__ dout,
-    T *__restrict__ dq, float *__restrict__ qdq, int T_len, int H, int reverse)
+    const T *__restrict__ k, const T *__restrict__ q, const T *__restrict__ dhT,
+    const TO *__restrict__ dout, T *__restrict__ dq, float *__restrict__ qdq, int T_len, int H, int reverse)
 {
     constexpr int DV = RV * 16, DK = DV;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -236,19 +236,44 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_dq_kernel(
         load_step(cur[0], step);
         compute(cur[0], step);
     }
+    // The last term of gla.py:263, sum_v dhT * hT per key feature, from the fp32 state this sweep ends with
+    // (the stored hidden_final is rounded to the element type).  Every d(log_fgate)_t is a sum over the
+    // steps s >= t, so the term is added to q*dq of the LAST step and reaches all of them through sweep 2's
+    // running sum.  The lane that adds it is the one that stored that q*dq.
+    {
+        const T *dp = dhT + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+        float f4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float d[RV], acc = 0.f;
+            load_vec<T, RV>(dp + (int64_t)i * DV, d);
+#pragma unroll
+            for (int j = 0; j < RV; ++j) acc += d[j] * S[i][j];
+            f4[i] = reduce_over_c(acc);
+        }
+        if (c == 0) {
+            float *lp = qdq + offK + (int64_t)(reverse ? 0 : T_len - 1) * strideK;
+            float w[4];
+            load_vec<float, 4>(lp, w);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w[i] += f4[i];
+            store_vec<float, 4>(lp, w);
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
 // backward, sweep 2 (against the forward's time direction), same tiling as sweep 1:
 //   dS = dcarry + q_t do_t^T ; dk_t = dS v_t ; dv_t = dS^T k_t ; dcarry = exp(g_t) * dS
 //   dg_t = sum_{s>=t}(q_s*dq_s - k_s*dk_s) + sum_v(dhT * hT)                      (gla.py:263)
+// (sweep 1 has added the last term to q*dq of the last step)
 // dv_t needs a sum over all DK rows, i.e. over the waves of the block: the per-wave partial sums of
 // TB steps are parked in LDS and combined once per TB steps.
 // ------------------------------------------------------------------------------------------------
 template <typename T, typename TO, int RV, int TB>
 __global__ __launch_bounds__(RV * 64) void recurrent_bwd_rev_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k,
-    const T *__restrict__ q, const T *__restrict__ hT, const T *__restrict__ dhT,
+    const T *__restrict__ q, const T *__restrict__ dhT,
     const TO *__restrict__ dout, T *__restrict__ dh0, float *__restrict__ dg, T *__restrict__ dv,
     T *__restrict__ dk, int T_len, int H, int reverse)
 {
@@ -260,19 +285,12 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_rev_kernel(
     const int dk0 = wave * 16 + a * 4, dv0 = c * RV;
     const int64_t bh = (int64_t)b * H + h;
 
-    float D[4][RV], fin[4], run[4];
+    float D[4][RV], run[4];   // run: sum over the later steps of q*dq - k*dk (sweep 1 put sum_v dhT*hT into the last q*dq)
     {
         const T *dp = dhT + bh * DK * DV + (int64_t)dk0 * DV + dv0;
-        const T *hp = hT + bh * DK * DV + (int64_t)dk0 * DV + dv0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            float hv[RV];
             load_vec<T, RV>(dp + (int64_t)i * DV, D[i]);
-            load_vec<T, RV>(hp + (int64_t)i * DV, hv);
-            float s = 0.f;
-#pragma unroll
-            for (int j = 0; j < RV; ++j) s += D[i][j] * hv[j];
-            fin[i] = reduce_over_c(s);
             run[i] = 0.f;
         }
     }
@@ -322,7 +340,7 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_rev_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             run[i] += s.w.get(i) - dkk[i] * s.k.get(i);
-            o[i] = run[i] + fin[i];
+            o[i] = run[i];
         }
         if (c == 0) {
             store_vec<T, 4>(dk + offK + t * strideK, dkk);
@@ -408,18 +426,18 @@ static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
     // sweep 1 of bf16 data at head dimension 64 runs on the matrix cores
     const bool stream1 = sizeof(T) == 2 && sizeof(TO) == 2 && DK == 64;
     if (stream1) {
-        int e = launch_recurrent_stream_dq(st, B, T_len, H, DK, reverse, h0, g, v, k, q, dout, dq, dg);
+        int e = launch_recurrent_stream_dq(st, B, T_len, H, DK, reverse, h0, g, v, k, q, dhT, dout, dq, dg);
         if (e) return e;
-        return launch_recurrent_stream_rev(st, B, T_len, H, DK, reverse, g, v, k, q, hT, dhT, dout, dh0, dg, dv, dk);
+        return launch_recurrent_stream_rev(st, B, T_len, H, DK, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
     }
 #define GLA_BWD_CASE(RV_, U_, TB_)                                                                      \
     do {                                                                                                \
         if (!stream1)                                                                                   \
             hipLaunchKernelGGL((recurrent_bwd_dq_kernel<T, TO, RV_, U_>), grid, block, 0, st,           \
                                (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,              \
-                               (const TO *)dout, (T *)dq, dg, T_len, H, reverse);                       \
+                               (const T *)dhT, (const TO *)dout, (T *)dq, dg, T_len, H, reverse);       \
         hipLaunchKernelGGL((recurrent_bwd_rev_kernel<T, TO, RV_, TB_>), grid, block, 0, st, g,          \
-                           (const T *)v, (const T *)k, (const T *)q, (const T *)hT, (const T *)dhT,     \
+                           (const T *)v, (const T *)k, (const T *)q, (const T *)dhT,                    \
                            (const TO *)dout, (T *)dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse);        \
     } while (0)
     switch (DV / 16) {

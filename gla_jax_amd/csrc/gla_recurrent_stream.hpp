@@ -11,14 +11,15 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
                                 const float *g, const void *v, const void *k, const void *q, void *hT,
                                 void *out);
 
-// Sweep 1 of the backward (bf16 everywhere): dq, and q*dq in fp32 into `qdq`.
+// Sweep 1 of the backward (bf16 everywhere): dq, and q*dq in fp32 into `qdq` (the last step's carries
+// sum_v dhT * (final state) on top).
 int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
-                               const float *g, const void *v, const void *k, const void *q, const void *dout,
-                               void *dq, float *qdq);
+                               const float *g, const void *v, const void *k, const void *q, const void *dhT,
+                               const void *dout, void *dq, float *qdq);
 
-// Sweep 2: dk, dv, dh0 and dlog_fgate (`dg` holds q*dq from sweep 1 on entry).
+// Sweep 2: dk, dv, dh0 and dlog_fgate (`dg` holds sweep 1's q*dq on entry).
 int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, const float *g,
-                                const void *v, const void *k, const void *q, const void *hT, const void *dhT,
+                                const void *v, const void *k, const void *q, const void *dhT,
                                 const void *dout, void *dh0, float *dg, void *dv, void *dk);
 
 }  // namespace gla

@@ -81,8 +81,8 @@ __device__ __forceinline__ void bwd_level(float (&p8)[8], float (&s8)[8], const 
 template <int C, int D>
 __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
     const BT *__restrict__ h0, const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k,
-    const BT *__restrict__ q, const BT *__restrict__ dout, BT *__restrict__ dq, float *__restrict__ qdq,
-    int T_len, int H, int reverse)
+    const BT *__restrict__ q, const BT *__restrict__ dhT, const BT *__restrict__ dout, BT *__restrict__ dq,
+    float *__restrict__ qdq, int T_len, int H, int reverse)
 {
     typedef BT T;
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16, RT = NT / NB;
@@ -373,6 +373,28 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
         __syncthreads();
         publish_state();
     }
+
+    // The last term of gla.py:263, sum_v dhT * hT per key feature, from the state this sweep ends with (just
+    // published as bf16 head + remainder: 16 bits of mantissa, where the stored hidden_final has 8).  Every
+    // d(log_fgate)_t is a sum over the steps s >= t, so the term is added to q*dq of the LAST step and
+    // reaches all of them through sweep 2's running sum.
+    __syncthreads();           // the published state and every q*dq row are in place
+    if (threadIdx.x < D) {
+        const int d = threadIdx.x;
+        const T *dp = dhT + bh * D * D + (int64_t)d * D;
+        float acc = 0.f;
+#pragma unroll 1
+        for (int j = 0; j < D; j += 8) {
+            float dv8[8], sh[8], sl[8];
+            unpack8(ld8(dp + j), dv8);
+            unpack8(ld8(Sh + d * LS + j), sh);
+            unpack8(ld8(Sl + d * LS + j), sl);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc += dv8[e] * (sh[e] + sl[e]);
+        }
+        float *lp = qdq + seq + (int64_t)(reverse ? 0 : T_len - 1) * rowstride + d;
+        *lp += acc;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -386,7 +408,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
 template <int C, int D>
 __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
     const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k, const BT *__restrict__ q,
-    const BT *__restrict__ hT, const BT *__restrict__ dhT, const BT *__restrict__ dout, BT *__restrict__ dh0,
+    const BT *__restrict__ dhT, const BT *__restrict__ dout, BT *__restrict__ dh0,
     float *__restrict__ dg, BT *__restrict__ dv, BT *__restrict__ dk, int T_len, int H, int reverse)
 {
     typedef BT T;
@@ -407,7 +429,6 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
     T *xs = DTl + D * LS;                          // [NB][2][16][XS] per-wave scratch
     float *rtab = reinterpret_cast<float *>(xs + NB * 2 * 16 * XS);   // [NB][D] exp(tau_m)
     float *dltab = rtab + NB * D;                  // [NB][D] sub-block sums of q*dq - k*dk
-    float *fintab = dltab + NB * D;                // [D] sum_v dhT * hT
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -450,11 +471,6 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
             }
     };
     publish();
-    for (int d = threadIdx.x; d < D; d += C * 4) {
-        float s = 0.f;
-        for (int j = 0; j < D; ++j) s += (float)dhT[bh * D * D + d * D + j] * (float)hT[bh * D * D + d * D + j];
-        fintab[d] = s;
-    }
     float run[NV];                           // sum over the later blocks of q*dq - k*dk, this lane's features
 #pragma unroll
     for (int i = 0; i < NV; ++i) run[i] = 0.f;
@@ -787,10 +803,10 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
         __syncthreads();                     // sub-block sums complete; every wave is done with the tiles
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            f32x8 o = ld8(fintab + 32 * ks + 8 * c), tot;
+            f32x8 o, tot;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                o.v[e] += qdq[8 * ks + e] + run[8 * ks + e];
+                o.v[e] = qdq[8 * ks + e] + run[8 * ks + e];
                 tot.v[e] = 0.f;
             }
 #pragma unroll
@@ -820,7 +836,8 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
 
 template <int C, int D>
 static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, const void *h0, const float *g,
-                     const void *v, const void *k, const void *q, const void *dout, void *dq, float *qdq)
+                     const void *v, const void *k, const void *q, const void *dhT, const void *dout, void *dq,
+                     float *qdq)
 {
     typedef BT T;
     constexpr int LS = TileGeom<T, D>::kStride;
@@ -831,41 +848,41 @@ static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, const
     if (int e = allow_lds((const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,
-                       (const T *)dout, (T *)dq, qdq, T_len, H, reverse);
+                       (const T *)dhT, (const T *)dout, (T *)dq, qdq, T_len, H, reverse);
     return launch_status();
 }
 
 template <int C, int D>
 static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, const float *g, const void *v,
-                      const void *k, const void *q, const void *hT, const void *dhT, const void *dout, void *dh0,
+                      const void *k, const void *q, const void *dhT, const void *dout, void *dh0,
                       float *dg, void *dv, void *dk)
 {
     typedef BT T;
     constexpr int LS = TileGeom<T, D>::kStride;
     constexpr int XS = 32 + 16 / (int)sizeof(T);
     const size_t lds = ((size_t)(3 * C + 4 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
-                       (size_t)(2 * (C / 16) + 1) * D * sizeof(float);
+                       (size_t)2 * (C / 16) * D * sizeof(float);
     auto kern = recurrent_stream_rev_kernel<C, D>;
     if (int e = allow_lds((const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
-    hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q, (const T *)hT,
+    hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
                        (const T *)dhT, (const T *)dout, (T *)dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse);
     return launch_status();
 }
 
 int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, const float *g,
-                                const void *v, const void *k, const void *q, const void *hT, const void *dhT,
+                                const void *v, const void *k, const void *q, const void *dhT,
                                 const void *dout, void *dh0, float *dg, void *dv, void *dk)
 {
-    if (D == 64) return launch_rev<64, 64>(st, B, T_len, H, reverse, g, v, k, q, hT, dhT, dout, dh0, dg, dv, dk);
+    if (D == 64) return launch_rev<64, 64>(st, B, T_len, H, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
     return GLA_ERR_UNSUPPORTED;
 }
 
 int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
-                               const float *g, const void *v, const void *k, const void *q, const void *dout,
-                               void *dq, float *qdq)
+                               const float *g, const void *v, const void *k, const void *q, const void *dhT,
+                               const void *dout, void *dq, float *qdq)
 {
-    if (D == 64) return launch_dq<64, 64>(st, B, T_len, H, reverse, h0, g, v, k, q, dout, dq, qdq);
+    if (D == 64) return launch_dq<64, 64>(st, B, T_len, H, reverse, h0, g, v, k, q, dhT, dout, dq, qdq);
     return GLA_ERR_UNSUPPORTED;
 }
 

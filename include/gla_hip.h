@@ -89,8 +89,10 @@ int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK,
 /* Replaces recurrent_gla_backward (gla.py:172-269, kernel gla.py:271-360): sweep 1 recomputes S_t
  * and forms dq_t; sweep 2 runs backwards for dk_t, dv_t and d(hidden_init); d(log_fgate) is the
  * reverse cumsum identity of gla.py:263 accumulated in fp32 inside sweep 2.  `hidden_final` is the
- * forward's residual (gla.py:169).  dlog_fgate doubles as the fp32 scratch that carries q*dq from
- * sweep 1 to sweep 2, so no workspace is needed.  dout has element type out_dtype. */
+ * forward's residual (gla.py:169); it is checked but not read: the term sum_v dhidden_final * hidden_final
+ * of gla.py:263 is formed from the fp32 state sweep 1 ends with, not from its stored rounding.
+ * dlog_fgate doubles as the fp32 scratch that carries q*dq from sweep 1 to sweep 2, so no workspace is
+ * needed.  dout has element type out_dtype. */
 int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
                       gla_dtype dtype, gla_dtype out_dtype, int reverse,
                       const void *hidden_init, const float *log_fgate, const void *value,

@@ -40,6 +40,23 @@ def test_recurrent_gla_matches_oracle(dtype, B, T, H, D, reverse):
         assert_close(name, to_np(got), e, tol, stored=st)
 
 
+@pytest.mark.parametrize("D", [32, 64])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_recurrent_gate_gradient_of_a_short_sequence(D, reverse):
+    """d(log_fgate) ends in sum_v dhidden_final * hidden_final (gla.py:263), the same for every step.  On a
+    short sequence with a large final state it dominates; it must come from the fp32 state of the backward's
+    first sweep (with the stored bf16 hidden_final it is off by 2^-9 of |dh.h|, 1.6e-2 of the gradient's norm
+    on this input).  Both the vector kernels (D=32) and the matrix-core kernels (D=64)."""
+    from gla_jax_amd import recurrent_gla
+    dtype = torch.bfloat16
+    (h0, g, v, k, q), dev = gpu_inputs(1, 13, 1, D, -2.0, seed=603, dtype=dtype)
+    dhT, dout = cotangents(h0, v, 103, dtype)
+    _, _, grads = run_fwd_bwd(recurrent_gla, dev, to_dev(dhT, dtype), to_dev(dout, dtype), dtype, reverse=reverse)
+    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=reverse)
+    err = to_np(grads[1]) - exp[1]
+    assert np.linalg.norm(err) <= 1e-3 * np.linalg.norm(exp[1])
+
+
 @pytest.mark.parametrize("reverse", [False, True])
 @pytest.mark.parametrize("T", [64, 200, 333])
 def test_recurrent_matrix_core_path_over_gate_regimes(T, reverse):
