@@ -419,8 +419,8 @@ static int launch_fwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
 template <typename T, typename TO>
 static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, int reverse,
                       const void *h0, const float *g, const void *v, const void *k, const void *q,
-                      const void *hT, const void *dhT, const void *dout, void *dh0, float *dg, void *dv,
-                      void *dk, void *dq)
+                      const void * /* hidden_final: recomputed in fp32 by sweep 1 */, const void *dhT,
+                      const void *dout, void *dh0, float *dg, void *dv, void *dk, void *dq)
 {
     dim3 grid(H, B), block(DK / 16 * 64);
     // sweep 1 of bf16 data at head dimension 64 runs on the matrix cores
