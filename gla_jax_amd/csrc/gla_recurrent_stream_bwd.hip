@@ -379,21 +379,26 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
     // d(log_fgate)_t is a sum over the steps s >= t, so the term is added to q*dq of the LAST step and
     // reaches all of them through sweep 2's running sum.
     __syncthreads();           // the published state and every q*dq row are in place
-    if (threadIdx.x < D) {
-        const int d = threadIdx.x;
-        const T *dp = dhT + bh * D * D + (int64_t)d * D;
+    static_assert(4 * D == C * 4, "four lanes per key feature");
+    {
+        const int d = threadIdx.x >> 2, part = threadIdx.x & 3;        // a quarter of the row each
+        const T *dp = dhT + bh * D * D + (int64_t)d * D + part * (D / 4);
         float acc = 0.f;
-#pragma unroll 1
-        for (int j = 0; j < D; j += 8) {
+#pragma unroll
+        for (int j = 0; j < D / 4; j += 8) {
             float dv8[8], sh[8], sl[8];
             unpack8(ld8(dp + j), dv8);
-            unpack8(ld8(Sh + d * LS + j), sh);
-            unpack8(ld8(Sl + d * LS + j), sl);
+            unpack8(ld8(Sh + d * LS + part * (D / 4) + j), sh);
+            unpack8(ld8(Sl + d * LS + part * (D / 4) + j), sl);
 #pragma unroll
             for (int e = 0; e < 8; ++e) acc += dv8[e] * (sh[e] + sl[e]);
         }
-        float *lp = qdq + seq + (int64_t)(reverse ? 0 : T_len - 1) * rowstride + d;
-        *lp += acc;
+        acc += dpp_f32<kDppQuadXor1>(acc);
+        acc += dpp_f32<kDppQuadXor2>(acc);
+        if (part == 0) {
+            float *lp = qdq + seq + (int64_t)(reverse ? 0 : T_len - 1) * rowstride + d;
+            *lp += acc;
+        }
     }
 }
 
