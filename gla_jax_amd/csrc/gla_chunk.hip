@@ -15,9 +15,11 @@ struct ChunkPlan {
 
 static size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-// The result does not depend on the chunk length (only its rounding does), so chunk sizes above the
-// largest compiled tile run with that tile; sizes below 32 tokens are not built (the leaf of the reference
-// needs 32 rows as well, gla.py:975-977).
+// The result does not depend on the chunk length (only its rounding does): chunk_size is checked as the
+// reference checks it, and the kernels then run with the largest compiled tile that divides T, whatever
+// size was asked for (at the headline shape a 64-token tile takes 1.5x, a 32-token tile 2.5x the time of
+// the 128-token one: twice or four times the chunk states).  Sizes below 32 tokens are refused: the leaf
+// of the reference needs 32 rows as well (gla.py:975-977).
 static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, int64_t chunk, int dtype,
                       ChunkPlan *plan)
 {
@@ -26,10 +28,10 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
     if (dtype != GLA_F32 && dtype != GLA_BF16) return GLA_ERR_DTYPE;
     if (DK != DV) return GLA_ERR_SHAPE;                      // gla.py:499
     if (!is_pow2(chunk) || T % chunk != 0) return GLA_ERR_CHUNK;   // gla.py:500, 674
-    int64_t C = chunk;
+    if (chunk < 32) return GLA_ERR_UNSUPPORTED;
     // largest tile built: 128 tokens for bf16, for fp32 (tiles twice as wide) 64 at D=64 and 32 at D=128
-    const int64_t cmax = dtype == GLA_BF16 ? 128 : (DK > 64 ? 32 : 64);
-    if (C > cmax) C = cmax;
+    int64_t C = dtype == GLA_BF16 ? 128 : (DK > 64 ? 32 : 64);
+    while (T % C != 0) C /= 2;                               // chunk >= 32 divides T, so this stops at 32 or above
     bool ok = false;
 #define GLA_PLAN_CASE(T_, C_, D_) \
     if (((dtype == GLA_BF16) == (sizeof(T_) == 2)) && C == C_ && DK == D_) ok = true;

@@ -155,7 +155,8 @@ def chunk_gla(hidden_init, log_fgate, value, key, query, chunk_size, block_size_
     """Chunk-wise parallel form of gated linear attention (gla.py:657-692).
 
     Same result as `recurrent_gla_naive` up to rounding.  `chunk_size` must be a power of two that
-    divides T (gla.py:500, 674).  `block_size_t`, `block_size_d`, `interpret`, `num_warps`,
+    divides T (gla.py:500, 674), at least 32; since the result does not depend on it, the kernels run
+    with the largest tile built that divides T, whatever size is given.  `block_size_t`, `block_size_d`, `interpret`, `num_warps`,
     `num_stages` tune the reference's Triton kernels; they are accepted for signature compatibility
     and have no effect here.  Differentiable in all five array arguments (gla.py:625)."""
     if interpret:

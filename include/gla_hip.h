@@ -104,8 +104,9 @@ int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK,
 
 /* Bytes of the `states` residual written by gla_chunk_fwd and read by gla_chunk_bwd: the
  * states before every chunk and after the last one, [B,H,T/C+1,DK,DV] in the element type, the analogue of
- * the reference's saved `state` (gla.py:548, 729; its last slice is hidden_final, gla.py:720-723).
- * Returns 0 for unsupported arguments. */
+ * the reference's saved `state` (gla.py:548, 729; its last slice is hidden_final, gla.py:720-723).  C is
+ * the tile the kernels run with: the largest one built that divides T (the result does not depend on the
+ * chunk length, so chunk_size is validated and otherwise not used).  Returns 0 for unsupported arguments. */
 size_t gla_chunk_states_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
                               int64_t chunk_size, gla_dtype dtype);
 /* Bytes of scratch needed by gla_chunk_fwd / gla_chunk_bwd.  Returns 0 for unsupported arguments. */
@@ -117,7 +118,7 @@ size_t gla_chunk_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK
 /* Replaces chunk_gla_forward (gla.py:483-550) and everything under it: the log-gate cumsum
  * (ops.py:234), compute_intra_contrib (gla.py:792-855) with compute_score (gla.py:964-1029),
  * compute_inter_contrib (gla.py:695-729) and the chunk state scan (ops.py:396).  Requires
- * DK == DV (gla.py:499), T % chunk_size == 0, chunk_size a power of two.  `states` receives the
+ * DK == DV (gla.py:499), T % chunk_size == 0, chunk_size a power of two >= 32.  `states` receives the
  * residual for the backward; pass NULL when no gradient will be taken. */
 int gla_chunk_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
                   int64_t chunk_size, gla_dtype dtype,

@@ -44,8 +44,11 @@ def test_chunk_plan_and_sizes():
     assert st == B * H * (n_chunks + 1) * D * D * 2      # states before every chunk + the final one
     ws = lib.gla_chunk_fwd_workspace_bytes(B, T, H, D, D, 128, _lib.GLA_BF16)
     assert ws >= B * H * n_chunks * (D * D * 4 + D * 4 + D * D * 2)
-    # chunk sizes above the largest tile reuse it; unsupported combinations report 0
+    # the tile is the largest one built that divides T, whatever chunk_size says; unsupported combinations report 0
     assert lib.gla_chunk_states_bytes(B, T, H, D, D, 256, _lib.GLA_BF16) == st
+    assert lib.gla_chunk_states_bytes(B, T, H, D, D, 32, _lib.GLA_BF16) == st
+    assert lib.gla_chunk_states_bytes(B, 64 * 65, H, D, D, 32, _lib.GLA_BF16) == B * H * (65 + 1) * D * D * 2
+    assert lib.gla_chunk_states_bytes(B, T, H, D, D, 16, _lib.GLA_BF16) == 0      # below the reference's own minimum
     assert lib.gla_chunk_states_bytes(B, T, H, D, D, 96, _lib.GLA_BF16) == 0      # not a power of two
     assert lib.gla_chunk_states_bytes(B, 100, H, D, D, 64, _lib.GLA_BF16) == 0    # does not divide T
     assert lib.gla_chunk_states_bytes(B, T, H, 128, 64, 128, _lib.GLA_BF16) == 0  # DK != DV

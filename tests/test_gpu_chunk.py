@@ -11,17 +11,20 @@ from tests.util import TOL, assert_close, cotangents, gpu_inputs, grad_kinds, to
 
 pytestmark = pytest.mark.gpu
 
+# The kernels run with the largest tile built (128, 64, 32 tokens; fp32: 64, 32 at D=64 and 32 at D=128) that
+# divides T, whatever chunk_size asks for: T picks the tile here.
 CASES = [
     # dtype, B, T, H, D, chunk, gate shift
     (torch.bfloat16, 2, 256, 2, 128, 128, 5.0),
-    (torch.bfloat16, 1, 512, 3, 64, 64, 5.0),
-    (torch.bfloat16, 2, 256, 1, 128, 64, 1.0),
+    (torch.bfloat16, 1, 448, 3, 64, 64, 5.0),       # 64-token tiles
+    (torch.bfloat16, 2, 192, 1, 128, 64, 1.0),      # 64-token tiles
     (torch.bfloat16, 1, 256, 2, 64, 128, 0.0),
-    (torch.bfloat16, 1, 128, 2, 64, 32, 3.0),
+    (torch.bfloat16, 1, 96, 2, 64, 32, 3.0),        # 32-token tiles
     (torch.bfloat16, 1, 512, 1, 128, 256, 5.0),     # chunk above the largest tile: same result
+    (torch.bfloat16, 1, 256, 2, 64, 32, 3.0),       # chunk below the tile that is used: same result
     (torch.float32, 1, 512, 2, 64, 64, 5.0),        # BASELINE configs[0]
-    (torch.float32, 2, 128, 1, 64, 32, 0.0),
-    (torch.bfloat16, 1, 256, 2, 128, 32, 2.0),      # the smallest tile at D=128
+    (torch.float32, 2, 96, 1, 64, 32, 0.0),         # fp32, 32-token tiles
+    (torch.bfloat16, 1, 160, 2, 128, 32, 2.0),      # the smallest tile at D=128
     (torch.float32, 1, 256, 2, 128, 128, 4.0),      # fp32 at D=128 runs on the 32-token tile
     (torch.bfloat16, 3, 128, 5, 128, 128, 3.0),     # a single chunk per sequence, odd batch and head counts
     (torch.bfloat16, 1, 64, 1, 64, 64, 3.0),
@@ -118,12 +121,13 @@ def test_chunk_size_and_concatenation_invariance():
     from gla_jax_amd import chunk_gla
     dtype = torch.float32
     (h0, g, v, k, q), dev = gpu_inputs(1, 256, 2, 64, 2.0, seed=31, dtype=dtype)
-    hA, oA = chunk_gla(*dev, 64)
-    hB, oB = chunk_gla(*dev, 32)
+    hA, oA = chunk_gla(*dev, 64)            # 256 tokens: 64-token tiles
+    hB, oB = chunk_gla(*dev, 32)            # the same tiles, whatever chunk_size says
     scale = oA.abs().max().item()
-    assert (oA - oB).abs().max().item() < 1e-4 * scale
-    h1, o1 = chunk_gla(dev[0], *[t[:, :128] for t in dev[1:]], 64)
-    h2, o2 = chunk_gla(h1, *[t[:, 128:] for t in dev[1:]], 64)
+    assert torch.equal(oA, oB) and torch.equal(hA, hB)
+    # the sequence cut at token 96: both pieces (96 and 160 tokens) run on 32-token tiles
+    h1, o1 = chunk_gla(dev[0], *[t[:, :96] for t in dev[1:]], 32)
+    h2, o2 = chunk_gla(h1, *[t[:, 96:] for t in dev[1:]], 32)
     assert (torch.cat([o1, o2], 1) - oA).abs().max().item() < 1e-4 * scale
     assert (h2 - hA).abs().max().item() < 1e-4 * hA.abs().max().item()
 
