@@ -75,17 +75,25 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     {
         float p[NV];
         D8 qf[KS], kf[KS];
+        // The gates come first and are scanned before q and k are requested: with all three in flight at
+        // once the 128 registers that let two workgroups share a CU do not suffice, and the spill of a
+        // freshly loaded row makes the wave wait for every request it has out.
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const int d0 = 32 * ks + 8 * c;
-            f32x8 gg = ld8(g + rowoff + d0);
+            f32x8 gg = ld8(g + rowoff + 32 * ks + 8 * c);
 #pragma unroll
             for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
-            qf[ks] = ld8(q + rowoff + d0);
-            kf[ks] = ld8(k + rowoff + d0);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            qf[ks] = ld8(q + rowoff + 32 * ks + 8 * c);
+            kf[ks] = ld8(k + rowoff + 32 * ks + 8 * c);
         }
 
-        subblock_forward<T, D>(p, qf, kf, g + rowoff, q + rowoff, k + rowoff, true, rtab + w * D, Kh + wrow,
+        subblock_forward<T, D, false, true>(p, qf, kf, g + rowoff, q + rowoff, k + rowoff, true, rtab + w * D, Kh + wrow,
                                w < NB - 1, nullptr, r, c, accD, qh);
     }
     // Values and the first state rows are requested only now: the registers above are free again, and

@@ -53,7 +53,8 @@ template <typename T4> __device__ __forceinline__ f32x4 mma_t_split(T4 ah, T4 al
 
 // PRECISE: the score products take their operands as head + remainder, for callers that promise fp32
 // arithmetic on bf16 inputs; kl_row must be given then.
-template <typename T, int D, bool PRECISE = false>
+// SCANNED: p already holds the inclusive prefix sums over the rows (the caller ran prefix_sum_rows).
+template <typename T, int D, bool PRECISE = false, bool SCANNED = false>
 __device__ __forceinline__ void subblock_forward(float (&p)[D / 4],
                                                  const typename FragTypes<T>::d8 (&qf)[D / 32],
                                                  const typename FragTypes<T>::d8 (&kf)[D / 32],
@@ -65,8 +66,10 @@ __device__ __forceinline__ void subblock_forward(float (&p)[D / 4],
     constexpr int KS = D / 32, NV = D / 4;
     typedef typename FragTypes<T>::d8 D8;
     // p = l_i; the totals travel through the wave's own table row (same-wave LDS accesses execute in order)
+    if constexpr (!SCANNED) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
+        for (int i = 0; i < NV; ++i) p[i] = prefix_sum_rows(p[i]);
+    }
     if (r == 15) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) st8(rt + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
