@@ -479,9 +479,9 @@ extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, 
     for (const void *p : ptrs)
         if (!gla::aligned16(p)) return GLA_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
-    // bf16 inputs at head dimension 64 run on the matrix cores, 64 steps per iteration
+    // bf16 inputs at head dimension 64 or 128 run on the matrix cores, 64 steps per iteration
     // (fp32 `out` is the recurrent_gla_naive flavour: it stays on the fp32 vector path below)
-    if (dtype == GLA_BF16 && out_dtype == GLA_BF16 && DK == 64)
+    if (dtype == GLA_BF16 && out_dtype == GLA_BF16 && (DK == 64 || DK == 128))
         return gla::launch_recurrent_stream_fwd<__bf16>(st, B, T, H, DK, reverse, hidden_init, log_fgate, value,
                                                         key, query, hidden_final, out);
     if (dtype == GLA_BF16 && out_dtype == GLA_BF16)

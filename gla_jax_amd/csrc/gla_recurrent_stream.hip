@@ -174,7 +174,12 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
         }
 
         // ---- out^T[dv][i] in slices of 32 output features: state term, then the score blocks --------
-#pragma unroll
+        // (a real loop at D = 128: one slice's temporaries live at a time.  Unrolled there, the slices at
+        // features 32 and 64 lost the last quarter of the state term; the published state was intact, so the
+        // reads were at fault: with the state tile above 51 KB of LDS the folded immediate offsets of the
+        // unrolled reads come close to or past the 16-bit limit.  With the slice offset in a register they
+        // stay small.)
+#pragma unroll(KS > 2 ? 1 : KS)
         for (int ks = 0; ks < KS; ++ks) {
             const int fo = 32 * ks;
             f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
@@ -258,6 +263,7 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
                                 void *out)
 {
     if (D == 64) return launch_one<TO, 64, 64>(st, B, T_len, H, reverse, h0, g, v, k, q, hT, out);
+    if (D == 128) return launch_one<TO, 64, 128>(st, B, T_len, H, reverse, h0, g, v, k, q, hT, out);
     return GLA_ERR_UNSUPPORTED;
 }
 

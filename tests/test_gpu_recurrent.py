@@ -57,15 +57,16 @@ def test_recurrent_gate_gradient_of_a_short_sequence(D, reverse):
     assert np.linalg.norm(err) <= 1e-3 * np.linalg.norm(exp[1])
 
 
+@pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("reverse", [False, True])
 @pytest.mark.parametrize("T", [64, 200, 333])
-def test_recurrent_matrix_core_path_over_gate_regimes(T, reverse):
-    """bf16 at D=64 runs 64 steps per iteration on the matrix cores: sequences that are not a multiple of
-    64 (padded steps), mild gates (one anchor per 16 steps) and hard ones (resets, the dyadic levels) in
-    the same sequence, both directions, forward and all gradients."""
+def test_recurrent_matrix_core_path_over_gate_regimes(T, reverse, D):
+    """bf16 at D=64 and D=128 runs 64 steps per iteration on the matrix cores: sequences that are not a
+    multiple of 64 (padded steps), mild gates (one anchor per 16 steps) and hard ones (resets, the dyadic
+    levels) in the same sequence, both directions, forward and all gradients."""
     from gla_jax_amd import recurrent_gla
     dtype = torch.bfloat16
-    (h0, g, v, k, q), dev = gpu_inputs(2, T, 2, 64, 1.0, seed=T + 7, dtype=dtype)
+    (h0, g, v, k, q), dev = gpu_inputs(2, T, 2, D, 1.0, seed=T + 7, dtype=dtype)
     g = g.copy()
     g[:, 5::37] = -200.0                       # hard resets at scattered positions
     g[:, T // 2:T // 2 + 4, :, ::2] = -60.0    # a hard stretch on every other feature
