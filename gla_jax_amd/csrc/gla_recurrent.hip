@@ -423,12 +423,13 @@ static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
                       const void *dout, void *dh0, float *dg, void *dv, void *dk, void *dq)
 {
     dim3 grid(H, B), block(DK / 16 * 64);
-    // sweep 1 of bf16 data at head dimension 64 runs on the matrix cores
-    const bool stream1 = sizeof(T) == 2 && sizeof(TO) == 2 && DK == 64;
+    // bf16 data at head dimension 64 runs both sweeps on the matrix cores, at 128 sweep 1 only
+    const bool stream1 = sizeof(T) == 2 && sizeof(TO) == 2 && (DK == 64 || DK == 128);
     if (stream1) {
         int e = launch_recurrent_stream_dq(st, B, T_len, H, DK, reverse, h0, g, v, k, q, dhT, dout, dq, dg);
         if (e) return e;
-        return launch_recurrent_stream_rev(st, B, T_len, H, DK, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
+        if (DK == 64)
+            return launch_recurrent_stream_rev(st, B, T_len, H, DK, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
     }
 #define GLA_BWD_CASE(RV_, U_, TB_)                                                                      \
     do {                                                                                                \

@@ -295,10 +295,23 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
         }
         __syncthreads();                     // tiles of this block and the published state are in place
 
+        // dA^T of the pairs with the earlier sub-blocks, [j][i] = v_j . do_i: they do not depend on the feature
+        T4 dah[NB], dal[NB];
+#pragma unroll
+        for (int J = 0; J < NB - 1; ++J) {
+            f32x4 da = {0.f, 0.f, 0.f, 0.f};
+            if (J < w) {
+#pragma unroll
+                for (int k2 = 0; k2 < KS; ++k2) da = mma_d(ld8(Vn + L.nat + 16 * J * LS + 32 * k2), dof[k2], da);
+            }
+            split4<T>(da, dah[J], dal[J]);
+        }
+
         // ---- dq chain: state term, then the earlier sub-blocks in ascending order, then the own one --------
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const int fo = 32 * ks;
+            if (KS > 2) __builtin_amdgcn_sched_barrier(0);   // one slice's operands at a time (register pressure)
             f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
             for (int k2 = 0; k2 < KS; ++k2) {
@@ -311,20 +324,14 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
 #pragma unroll
             for (int J = 0; J < NB - 1; ++J) {
                 if (J < w) {
-                    // dA^T of the pair: [j][i] = v_j . do_i
-                    f32x4 da = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int k2 = 0; k2 < KS; ++k2)
-                        da = mma_d(ld8(Vn + L.nat + 16 * J * LS + 32 * k2), dof[k2], da);
-                    T4 dah, dal;
-                    split4<T>(da, dah, dal);
                     f32x8 rr = ld8(rtab + J * D + fo + 8 * c);
 #pragma unroll
                     for (int tt = 0; tt < 2; ++tt) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) acc[tt][e] *= rr.v[4 * tt + e];
                         acc[tt] = mma_t_split(lds_tr4(Kh + L.k4 + fo + 4 * tt + 16 * J * LS, LS),
-                                              lds_tr4(Kl + L.k4 + fo + 4 * tt + 16 * J * LS, LS), dah, dal, acc[tt]);
+                                              lds_tr4(Kl + L.k4 + fo + 4 * tt + 16 * J * LS, LS), dah[J], dal[J],
+                                              acc[tt]);
                     }
                 }
             }
@@ -379,22 +386,23 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
     // d(log_fgate)_t is a sum over the steps s >= t, so the term is added to q*dq of the LAST step and
     // reaches all of them through sweep 2's running sum.
     __syncthreads();           // the published state and every q*dq row are in place
-    static_assert(4 * D == C * 4, "four lanes per key feature");
     {
-        const int d = threadIdx.x >> 2, part = threadIdx.x & 3;        // a quarter of the row each
-        const T *dp = dhT + bh * D * D + (int64_t)d * D + part * (D / 4);
+        constexpr int LPF = C * 4 / D;                                   // lanes per key feature: 4 or 2
+        static_assert(LPF == 4 || LPF == 2, "a quad or a pair of lanes shares a key feature");
+        const int d = threadIdx.x / LPF, part = threadIdx.x % LPF;       // each takes D / LPF of the row
+        const T *dp = dhT + bh * D * D + (int64_t)d * D + part * (D / LPF);
         float acc = 0.f;
 #pragma unroll
-        for (int j = 0; j < D / 4; j += 8) {
+        for (int j = 0; j < D / LPF; j += 8) {
             float dv8[8], sh[8], sl[8];
             unpack8(ld8(dp + j), dv8);
-            unpack8(ld8(Sh + d * LS + part * (D / 4) + j), sh);
-            unpack8(ld8(Sl + d * LS + part * (D / 4) + j), sl);
+            unpack8(ld8(Sh + d * LS + part * (D / LPF) + j), sh);
+            unpack8(ld8(Sl + d * LS + part * (D / LPF) + j), sl);
 #pragma unroll
             for (int e = 0; e < 8; ++e) acc += dv8[e] * (sh[e] + sl[e]);
         }
         acc += dpp_f32<kDppQuadXor1>(acc);
-        acc += dpp_f32<kDppQuadXor2>(acc);
+        if (LPF == 4) acc += dpp_f32<kDppQuadXor2>(acc);
         if (part == 0) {
             float *lp = qdq + seq + (int64_t)(reverse ? 0 : T_len - 1) * rowstride + d;
             *lp += acc;
@@ -888,6 +896,7 @@ int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, i
                                const void *dout, void *dq, float *qdq)
 {
     if (D == 64) return launch_dq<64, 64>(st, B, T_len, H, reverse, h0, g, v, k, q, dhT, dout, dq, qdq);
+    if (D == 128) return launch_dq<64, 128>(st, B, T_len, H, reverse, h0, g, v, k, q, dhT, dout, dq, qdq);
     return GLA_ERR_UNSUPPORTED;
 }
 
