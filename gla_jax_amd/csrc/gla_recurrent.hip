@@ -428,8 +428,7 @@ static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
     if (stream1) {
         int e = launch_recurrent_stream_dq(st, B, T_len, H, DK, reverse, h0, g, v, k, q, dhT, dout, dq, dg);
         if (e) return e;
-        if (DK == 64)
-            return launch_recurrent_stream_rev(st, B, T_len, H, DK, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
+        return launch_recurrent_stream_rev(st, B, T_len, H, DK, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
     }
 #define GLA_BWD_CASE(RV_, U_, TB_)                                                                      \
     do {                                                                                                \

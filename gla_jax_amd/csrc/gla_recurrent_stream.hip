@@ -132,7 +132,6 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
                 kf[ks] = kN[ks];
                 st8(Vn + wrow + 32 * ks, vN[ks]);
             }
-            if (n + 1 < N) fetch(n + 1);
             subblock_forward<T, D, true>(p, qf, kf, g + row, q + row, k + row, valid, rtab + w * D, Kh + wrow, true,
                                    Kl + wrow, r, c, accD, qh);
         }
@@ -210,6 +209,10 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
             for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
             if (valid) OutPack<TO>::store(out + row + fo + 8 * c, o);
         }
+
+        // The next block's rows are requested only here: the registers that receive them are not held through
+        // the score and output phases above, and the update below is long enough for them to arrive.
+        if (n + 1 < N) fetch(n + 1);
 
         // ---- state update: S <- S e^{tau_J} + V_J^T (k e^{tau_J - l})_J over the sub-blocks in order ------
 #pragma unroll

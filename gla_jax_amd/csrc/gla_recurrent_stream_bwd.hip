@@ -186,7 +186,6 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
                 dof[ks] = dN[ks];
                 st8(Vn + wrow + 32 * ks, vf[ks]);
             }
-            if (n + 1 < N) fetch(n + 1);
 
             // dAt[e] = dA[i = r][j = 4c+e], dAn[e] = dA[i = 4c+e][j = r]  (dA = dO V^T: exact products of bf16)
             f32x4 dAn = {0.f, 0.f, 0.f, 0.f}, dAt = {0.f, 0.f, 0.f, 0.f};
@@ -359,6 +358,9 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
             }
         }
 
+        // the next block's rows are requested only here (see sweep 2)
+        if (n + 1 < N) fetch(n + 1);
+
         // ---- state update: S <- S e^{tau_J} + V_J^T (k e^{tau_J - l})_J over the sub-blocks in order ------
 #pragma unroll
         for (int J = 0; J < NB; ++J) {
@@ -435,9 +437,9 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
     T *tO = reinterpret_cast<T *>(smem);           // [C][LS]  dout
     T *Qh = tO + C * LS;                           // [C][LS]  q * exp(l_i), bf16 head
     T *Ql = Qh + C * LS;                           // [C][LS]  ... and remainder
-    T *DNh = Ql + C * LS;                          // [D][LS]  dS' as [dk][dv], head / remainder
-    T *DNl = DNh + D * LS;
-    T *DTh = DNl + D * LS;                         // [D][LS]  dS' as [dv][dk], head / remainder
+    // dS' is kept in ONE orientation, [dv][dk] (head / remainder): the product that contracts over dk reads its
+    // rows, the one that contracts over dv reads it transposed, 16 dv rows per MFMA.
+    T *DTh = Ql + C * LS;                          // [D][LS]
     T *DTl = DTh + D * LS;
     T *xs = DTl + D * LS;                          // [NB][2][16][XS] per-wave scratch
     float *rtab = reinterpret_cast<float *>(xs + NB * 2 * 16 * XS);   // [NB][D] exp(tau_m)
@@ -476,11 +478,6 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                 const int dk0 = 16 * (w + i * NB) + 4 * c, dvc = 16 * nt + r;
                 *reinterpret_cast<T4 *>(DTh + dvc * LS + dk0) = hi;
                 *reinterpret_cast<T4 *>(DTl + dvc * LS + dk0) = lo;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    DNh[(dk0 + e) * LS + dvc] = hi[e];
-                    DNl[(dk0 + e) * LS + dvc] = lo[e];
-                }
             }
     };
     publish();
@@ -543,7 +540,6 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                 dof[ks] = dN[ks];
                 st8(tO + wrow + 32 * ks, dof[ks]);
             }
-            if (n > 0) fetch(n - 1);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 dAn = mma_d(dof[ks], vf[ks], dAn);
@@ -758,12 +754,19 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
             // -- dk slice: dS' v first, then the later sub-blocks in descending order
             {
                 f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+                // (dS' v)[dk][j] = sum_dv dS'[dk][dv] v_j[dv]: 16 dv rows per step, read transposed.  Step (k2,
+                // half) contracts over dv = 32 k2 + 8 c + 4 half + m, which is what lane (j, c) holds of v_j.
 #pragma unroll
                 for (int k2 = 0; k2 < KS; ++k2) {
 #pragma unroll
-                    for (int tt = 0; tt < 2; ++tt) {
-                        acc[tt] = mma_d(ld8(DNl + L.own + (fo + 4 * tt) * LS + 32 * k2), vf[k2], acc[tt]);
-                        acc[tt] = mma_d(ld8(DNh + L.own + (fo + 4 * tt) * LS + 32 * k2), vf[k2], acc[tt]);
+                    for (int half = 0; half < 2; ++half) {
+                        const T4 vb = half ? __builtin_shufflevector(vf[k2], vf[k2], 4, 5, 6, 7)
+                                           : __builtin_shufflevector(vf[k2], vf[k2], 0, 1, 2, 3);
+#pragma unroll
+                        for (int tt = 0; tt < 2; ++tt) {
+                            acc[tt] = mma_t(lds_tr4(DTl + L.k8 + (32 * k2 + 4 * half) * LS + fo + 4 * tt, LS), vb, acc[tt]);
+                            acc[tt] = mma_t(lds_tr4(DTh + L.k8 + (32 * k2 + 4 * half) * LS + fo + 4 * tt, LS), vb, acc[tt]);
+                        }
                     }
                 }
 #pragma unroll
@@ -794,6 +797,10 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                 if (r == 0) st8(dltab + w * D + fo + 8 * c, sfx);
             }
         }
+
+        // The next block's rows are requested only here: the registers that receive them are not held through
+        // the chains above, and the update below is long enough for them to arrive.
+        if (n > 0) fetch(n - 1);
 
         // ---- dS <- dS r_I + (q e^{l})_I^T dO_I over the sub-blocks, last first ---------------------------
 #pragma unroll
@@ -873,7 +880,7 @@ static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, cons
     typedef BT T;
     constexpr int LS = TileGeom<T, D>::kStride;
     constexpr int XS = 32 + 16 / (int)sizeof(T);
-    const size_t lds = ((size_t)(3 * C + 4 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
+    const size_t lds = ((size_t)(3 * C + 2 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
                        (size_t)2 * (C / 16) * D * sizeof(float);
     auto kern = recurrent_stream_rev_kernel<C, D>;
     if (int e = allow_lds((const void *)kern, lds)) return e;
@@ -888,6 +895,7 @@ int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, 
                                 const void *dout, void *dh0, float *dg, void *dv, void *dk)
 {
     if (D == 64) return launch_rev<64, 64>(st, B, T_len, H, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
+    if (D == 128) return launch_rev<64, 128>(st, B, T_len, H, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
     return GLA_ERR_UNSUPPORTED;
 }
 
