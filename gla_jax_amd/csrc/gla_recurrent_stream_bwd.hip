@@ -485,7 +485,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
 #pragma unroll
     for (int i = 0; i < NV; ++i) run[i] = 0.f;
 
-    f32x8 gN[KS], wN[KS];
+    f32x8 gN[KS];
     D8 qN[KS], kN[KS], vN[KS], dN[KS];
     bool validN;
     int64_t rowN;
@@ -497,7 +497,6 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             gN[ks] = ld8(g + rowN + 32 * ks + 8 * c);
-            wN[ks] = ld8(dg + rowN + 32 * ks + 8 * c);
             qN[ks] = ld8(q + rowN + 32 * ks + 8 * c);
             kN[ks] = ld8(k + rowN + 32 * ks + 8 * c);
             vN[ks] = ld8(v + rowN + 32 * ks + 8 * c);
@@ -523,7 +522,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                 float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    gN[ks] = wN[ks] = pack8<float>(z);
+                    gN[ks] = pack8<float>(z);
                     qN[ks] = kN[ks] = vN[ks] = dN[ks] = pack8<T>(z);
                 }
             }
@@ -532,7 +531,6 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     p[8 * ks + e] = gN[ks].v[e] * kLog2e;
-                    qdq[8 * ks + e] = wN[ks].v[e];
                 }
                 qf[ks] = qN[ks];
                 kf[ks] = kN[ks];
@@ -685,6 +683,14 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
             for (int e = 0; e < 4; ++e) Aown[e] += (4 * c + e == r) ? dot : 0.f;   // A_ii = q_i.k_i (gla.py:983)
         }
         __syncthreads();                     // tiles of this block and the published dS' are in place
+        // q*dq of the block's rows (sweep 1 left it in the d(log_fgate) buffer) is requested here, not with the
+        // rest of the block: it is needed last, and is not held through the work above
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            f32x8 t = ld8(dg + row + 32 * ks + 8 * c);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qdq[8 * ks + e] = valid ? t.v[e] : 0.f;
+        }
 
         // ---- score blocks of the later sub-blocks: A_Ij (key side walked up by r_I) and dA_Ij ----------
         T4 Ach[NB], Acl[NB], dAh[NB], dAl[NB];
