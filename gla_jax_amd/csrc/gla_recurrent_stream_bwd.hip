@@ -444,6 +444,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
     T *xs = DTl + D * LS;                          // [NB][2][16][XS] per-wave scratch
     float *rtab = reinterpret_cast<float *>(xs + NB * 2 * 16 * XS);   // [NB][D] exp(tau_m)
     float *dltab = rtab + NB * D;                  // [NB][D] sub-block sums of q*dq - k*dk
+    float *runtab = dltab + NB * D;                // [2][D]  sum over the later blocks of q*dq - k*dk, double-buffered
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -481,9 +482,9 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
             }
     };
     publish();
-    float run[NV];                           // sum over the later blocks of q*dq - k*dk, this lane's features
-#pragma unroll
-    for (int i = 0; i < NV; ++i) run[i] = 0.f;
+    // the running sum over the later blocks is the same for all rows: it lives in LDS, block n reads buffer
+    // n & 1 and wave 0 writes the other one, so readers and the writer never meet between two barriers
+    for (int d = threadIdx.x; d < 2 * D; d += C * 4) runtab[d] = 0.f;
 
     f32x8 gN[KS];
     D8 qN[KS], kN[KS], vN[KS], dN[KS];
@@ -829,12 +830,9 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
         __syncthreads();                     // sub-block sums complete; every wave is done with the tiles
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            f32x8 o, tot;
+            f32x8 o, tot = ld8(runtab + (n & 1) * D + 32 * ks + 8 * c);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                o.v[e] = qdq[8 * ks + e] + run[8 * ks + e];
-                tot.v[e] = 0.f;
-            }
+            for (int e = 0; e < 8; ++e) o.v[e] = qdq[8 * ks + e] + tot.v[e];
 #pragma unroll
             for (int m = 0; m < NB; ++m) {
                 f32x8 t = ld8(dltab + m * D + 32 * ks + 8 * c);
@@ -844,8 +842,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                     tot.v[e] += t.v[e];
                 }
             }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) run[8 * ks + e] += tot.v[e];
+            if (w == 0 && r == 0) st8(runtab + ((n & 1) ^ 1) * D + 32 * ks + 8 * c, tot);
             if (valid) st8(dg + row + 32 * ks + 8 * c, o);
         }
         publish();
@@ -887,7 +884,7 @@ static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, cons
     constexpr int LS = TileGeom<T, D>::kStride;
     constexpr int XS = 32 + 16 / (int)sizeof(T);
     const size_t lds = ((size_t)(3 * C + 2 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
-                       (size_t)2 * (C / 16) * D * sizeof(float);
+                       (size_t)(2 * (C / 16) + 2) * D * sizeof(float);
     auto kern = recurrent_stream_rev_kernel<C, D>;
     if (int e = allow_lds((const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
