@@ -173,12 +173,12 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
         }
 
         // ---- out^T[dv][i] in slices of 32 output features: state term, then the score blocks --------
-        // (a real loop at D = 128: one slice's temporaries live at a time.  Unrolled there, the slices at
-        // features 32 and 64 lost the last quarter of the state term; the published state was intact, so the
-        // reads were at fault: with the state tile above 51 KB of LDS the folded immediate offsets of the
-        // unrolled reads come close to or past the 16-bit limit.  With the slice offset in a register they
-        // stay small.)
-#pragma unroll(KS > 2 ? 1 : KS)
+        // (a real loop at D = 128: one slice's temporaries live at a time.  The fully unrolled form was also
+        // WRONG there: the slices at features 32 and 64 lost the key features 96..127 of the state term,
+        // with the published state intact and every immediate offset of the reads in range; the cause was
+        // not found, so the unrolled form stays out for D = 128.)
+        constexpr int kSliceUnroll = KS > 2 ? 1 : KS;
+#pragma unroll kSliceUnroll
         for (int ks = 0; ks < KS; ++ks) {
             const int fo = 32 * ks;
             f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
