@@ -37,8 +37,11 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
     TO *__restrict__ out, int T_len, int H, int reverse)
 {
     typedef __bf16 T;
-    constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16, RT = NT / NB;
-    static_assert(NT % NB == 0, "every wave owns the same number of state row tiles");
+    constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16;
+    // The NT x NT state tiles are split evenly over the waves: a wave owns RT tile rows (dv) and NTW of the
+    // NT tile columns (dk).  With more waves than tile rows, G waves share a row and split its columns.
+    constexpr int G = NB > NT ? NB / NT : 1, RT = NB > NT ? 1 : NT / NB, NTW = NT / G, NDV = NB / G;
+    static_assert(NT * NT % NB == 0 && NDV * RT == NT && NTW * G == NT, "the state tiles split evenly over the waves");
     constexpr int LS = TileGeom<T, D>::kStride;
     typedef typename FragTypes<T>::d8 D8;
     typedef typename FragTypes<T>::t4 T4;
@@ -61,28 +64,29 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
     const int ptl = plain_tr_lane<T>(LS);
     const int wrow = 16 * w * LS + L.nat;          // this lane's row of a [token][feature] tile
     const int N = (T_len + C - 1) / C;
+    const int wv = w % NDV, nt0 = (w / NDV) * NTW;   // the wave's tile rows are wv + i NDV, its tile columns nt0 + j
 
-    // state: S[i][nt][e] = state[dk = 16nt + r][dv = 16(w + i NB) + 4c + e]  (accumulator layout of a
+    // state: S[i][j][e] = state[dk = 16(nt0 + j) + r][dv = 16(wv + i NDV) + 4c + e]  (accumulator layout of a
     // (dv x dk) product tile)
-    f32x4 S[RT][NT];
+    f32x4 S[RT][NTW];
 #pragma unroll
     for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
+        for (int nt = 0; nt < NTW; ++nt) {
             float t4[4];
-            load_vec<T, 4>(h0 + bh * D * D + (int64_t)(16 * nt + r) * D + 16 * (w + i * NB) + 4 * c, t4);
+            load_vec<T, 4>(h0 + bh * D * D + (int64_t)(16 * (nt0 + nt) + r) * D + 16 * (wv + i * NDV) + 4 * c, t4);
             S[i][nt] = f32x4{t4[0], t4[1], t4[2], t4[3]};
         }
     auto publish_state = [&]() {
 #pragma unroll
         for (int i = 0; i < RT; ++i)
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+            for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const T hi = (T)S[i][nt][e];
-                    St[(16 * (w + i * NB) + 4 * c + e) * LS + 16 * nt + r] = hi;
-                    Sl[(16 * (w + i * NB) + 4 * c + e) * LS + 16 * nt + r] = (T)(S[i][nt][e] - (float)hi);
+                    St[(16 * (wv + i * NDV) + 4 * c + e) * LS + 16 * (nt0 + nt) + r] = hi;
+                    Sl[(16 * (wv + i * NDV) + 4 * c + e) * LS + 16 * (nt0 + nt) + r] = (T)(S[i][nt][e] - (float)hi);
                 }
     };
     publish_state();
@@ -217,18 +221,18 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
         // ---- state update: S <- S e^{tau_J} + V_J^T (k e^{tau_J - l})_J over the sub-blocks in order ------
 #pragma unroll
         for (int J = 0; J < NB; ++J) {
-            float rr[NT];
+            float rr[NTW];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) rr[nt] = rtab[J * D + 16 * nt + r];
+            for (int nt = 0; nt < NTW; ++nt) rr[nt] = rtab[J * D + 16 * (nt0 + nt) + r];
 #pragma unroll
             for (int i = 0; i < RT; ++i) {
-                auto va = lds_tr4(Vn + ptl + 16 * J * LS + 16 * (w + i * NB), LS);
+                auto va = lds_tr4(Vn + ptl + 16 * J * LS + 16 * (wv + i * NDV), LS);
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
+                for (int nt = 0; nt < NTW; ++nt) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) S[i][nt][e] *= rr[nt];
-                    S[i][nt] = mma_t(va, lds_tr4(Kl + ptl + 16 * J * LS + 16 * nt, LS), S[i][nt]);
-                    S[i][nt] = mma_t(va, lds_tr4(Kh + ptl + 16 * J * LS + 16 * nt, LS), S[i][nt]);
+                    S[i][nt] = mma_t(va, lds_tr4(Kl + ptl + 16 * J * LS + 16 * (nt0 + nt), LS), S[i][nt]);
+                    S[i][nt] = mma_t(va, lds_tr4(Kh + ptl + 16 * J * LS + 16 * (nt0 + nt), LS), S[i][nt]);
                 }
             }
         }
@@ -239,9 +243,9 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
 #pragma unroll
     for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
+        for (int nt = 0; nt < NTW; ++nt) {
             float t4[4] = {S[i][nt][0], S[i][nt][1], S[i][nt][2], S[i][nt][3]};
-            store_vec<T, 4>(hT + bh * D * D + (int64_t)(16 * nt + r) * D + 16 * (w + i * NB) + 4 * c, t4);
+            store_vec<T, 4>(hT + bh * D * D + (int64_t)(16 * (nt0 + nt) + r) * D + 16 * (wv + i * NDV) + 4 * c, t4);
         }
 }
 
@@ -265,7 +269,7 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
                                 const float *g, const void *v, const void *k, const void *q, void *hT,
                                 void *out)
 {
-    if (D == 64) return launch_one<TO, 64, 64>(st, B, T_len, H, reverse, h0, g, v, k, q, hT, out);
+    if (D == 64) return launch_one<TO, 128, 64>(st, B, T_len, H, reverse, h0, g, v, k, q, hT, out);
     if (D == 128) return launch_one<TO, 64, 128>(st, B, T_len, H, reverse, h0, g, v, k, q, hT, out);
     return GLA_ERR_UNSUPPORTED;
 }
