@@ -24,7 +24,7 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
                       ChunkPlan *plan)
 {
     if (B <= 0 || T <= 0 || H <= 0 || DK <= 0 || DV <= 0) return GLA_ERR_SHAPE;
-    if (B > 65535 || H > 65535 || T > (1 << 30)) return GLA_ERR_SHAPE;
+    if (B > 65535 || H > 65535 || T > (1 << 30) || B * H > 0x7fffffffLL) return GLA_ERR_SHAPE;   // grid limits
     if (dtype != GLA_F32 && dtype != GLA_BF16) return GLA_ERR_DTYPE;
     if (DK != DV) return GLA_ERR_SHAPE;                      // gla.py:499
     if (!is_pow2(chunk) || T % chunk != 0) return GLA_ERR_CHUNK;   // gla.py:500, 674

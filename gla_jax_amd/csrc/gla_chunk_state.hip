@@ -149,8 +149,12 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ h
 {
     typedef typename Pair<T>::type P2;
     constexpr int TPD = D / 32;
-    const int bh = blockIdx.y;
-    const int tile_v = blockIdx.x / TPD, tile_k = blockIdx.x % TPD;
+    // (b,h) runs along x, the 32x32 tiles along y: workgroups are dealt to the 8 XCDs in x-major order, so when
+    // the number of (b,h) pairs is a multiple of 8 all tiles of one state meet in ONE L2.  A tile row is half a
+    // 128-byte line of the bf16 states: the halves written by neighbouring tiles are then merged there and
+    // leave as whole lines.
+    const int bh = blockIdx.x;
+    const int tile_v = blockIdx.y / TPD, tile_k = blockIdx.y % TPD;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ti = lane >> 3, tj = lane & 7;
     const int dv0 = 32 * tile_v + 16 * (wave >> 1) + 2 * ti;
@@ -255,8 +259,8 @@ template <typename T, int D>
 int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hin, const float *prodT,
                       const float *decay, void *statesT, void *statesN, void *hout, int tail)
 {
-    dim3 grid((D / 32) * (D / 32), BH), block(256);
-    if ((int64_t)grid.x * BH >= 256) {
+    dim3 grid(BH, (D / 32) * (D / 32)), block(256);
+    if ((int64_t)grid.y * BH >= 256) {
         hipLaunchKernelGGL((chunk_scan_kernel<T, D, 4>), grid, block, 0, st, (const T *)hin, prodT, decay,
                            (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
     } else {
