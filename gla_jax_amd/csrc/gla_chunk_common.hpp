@@ -174,17 +174,6 @@ template <typename T> __device__ __forceinline__ TrLane<T> make_tr_lane(int stri
     }
     return t;
 }
-// compile-time part of a transposed read: band starting at row `krow`, feature tile t
-__host__ __device__ constexpr int tr_const(int krow, int t, int stride)
-{
-    return krow * stride + 32 * (t >> 1) + 4 * (t & 1);
-}
-// compile-time part of a natural read of row pi(t, .) at feature offset f
-__host__ __device__ constexpr int own_const(int t, int f, int stride)
-{
-    return (32 * (t >> 1) + 4 * (t & 1)) * stride + f;
-}
-
 __device__ __forceinline__ bf16x4 lds_tr4(const __bf16 *p, int stride)
 {
     (void)stride;
@@ -275,16 +264,6 @@ __device__ __forceinline__ float reduce_over_cgroups(float x)
 {
     x += shfl_xor_f32(x, 16);
     x += shfl_xor_f32(x, 32);
-    return x;
-}
-
-// Sum over the 16 token rows of the wave (lanes of one DPP row); every lane gets the total.
-__device__ __forceinline__ float reduce_over_rows(float x)
-{
-    x += dpp_f32<kDppQuadXor1>(x);
-    x += dpp_f32<kDppQuadXor2>(x);
-    x += dpp_f32<kDppRowHalfMirror>(x);
-    x += dpp_f32<kDppRowMirror>(x);
     return x;
 }
 
