@@ -140,8 +140,8 @@ template <> struct Pair<float> { typedef f32x2 type; };
 
 // U = chunks whose inputs are in flight per thread: 4 when the grid fills the machine, 32 when few (b,h)
 // pairs leave it to the single thread to keep the memory system busy (long sequences, small batch).
-template <typename T, int D, int U>
-__global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ hin,
+template <typename T, int D, int U, int WPB = 4>
+__global__ __launch_bounds__(64 * WPB) void chunk_scan_kernel(const T *__restrict__ hin,
                                                          const float *__restrict__ prodT,
                                                          const float *__restrict__ decay,
                                                          T *__restrict__ statesT, T *__restrict__ statesN,
@@ -154,8 +154,10 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(const T *__restrict__ h
     // 128-byte line of the bf16 states: the halves written by neighbouring tiles are then merged there and
     // leave as whole lines.
     const int bh = blockIdx.x;
-    const int tile_v = blockIdx.y / TPD, tile_k = blockIdx.y % TPD;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // WPB waves per block: a block is a 32x32 tile (WPB = 4) or one of its 16x16 quarters (WPB = 1)
+    const int wg = blockIdx.y * WPB + (threadIdx.x >> 6);
+    const int tile_v = (wg >> 2) / TPD, tile_k = (wg >> 2) % TPD;
+    const int lane = threadIdx.x & 63, wave = wg & 3;
     const int ti = lane >> 3, tj = lane & 7;
     const int dv0 = 32 * tile_v + 16 * (wave >> 1) + 2 * ti;
     const int dk0 = 32 * tile_k + 16 * (wave & 1) + 2 * tj;
@@ -264,7 +266,9 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hi
         hipLaunchKernelGGL((chunk_scan_kernel<T, D, 4>), grid, block, 0, st, (const T *)hin, prodT, decay,
                            (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
     } else {
-        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 32>), grid, block, 0, st, (const T *)hin, prodT, decay,
+        // few (b,h) pairs: one wave per block, so that the quarters of a tile spread over four CUs
+        grid.y *= 4;
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 32, 1>), grid, dim3(64), 0, st, (const T *)hin, prodT, decay,
                            (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
     }
     return launch_status();
