@@ -130,18 +130,20 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     }
 }
 
-// One thread = a 2x2 patch of the state, one wave = a 16x16 sub-tile (8x8 lanes), one block = a 32x32
-// tile, walked over the chunks in registers.  The running state is written per chunk in BOTH
-// orientations ([dv][dk] for products contracting over dk, [dk][dv] for products contracting over dv);
-// with 8x8 lanes of 2x2 patches every store instruction fills whole 32-byte sectors either way.
+// One thread = a 2x2 patch of the state, one block = one wave = a 16x16 tile (8x8 lanes), walked over the
+// chunks in registers.  The running state is written per chunk in BOTH orientations ([dv][dk] for products
+// contracting over dk, [dk][dv] for products contracting over dv); with 8x8 lanes of 2x2 patches every
+// store instruction fills whole 32-byte sectors either way.  Single-wave blocks spread a state over as many
+// CUs as possible: with four-wave blocks the headline shape left a third of the chip with half the work
+// (20 -> 18 us), and 8 sequences used 128 CUs (77 -> 60 us).
 template <typename T> struct Pair;
 template <> struct Pair<__bf16> { typedef bf16x2 type; };
 template <> struct Pair<float> { typedef f32x2 type; };
 
 // U = chunks whose inputs are in flight per thread: 4 when the grid fills the machine, 32 when few (b,h)
 // pairs leave it to the single thread to keep the memory system busy (long sequences, small batch).
-template <typename T, int D, int U, int WPB = 4>
-__global__ __launch_bounds__(64 * WPB) void chunk_scan_kernel(const T *__restrict__ hin,
+template <typename T, int D, int U>
+__global__ __launch_bounds__(64) void chunk_scan_kernel(const T *__restrict__ hin,
                                                          const float *__restrict__ prodT,
                                                          const float *__restrict__ decay,
                                                          T *__restrict__ statesT, T *__restrict__ statesN,
@@ -154,10 +156,8 @@ __global__ __launch_bounds__(64 * WPB) void chunk_scan_kernel(const T *__restric
     // 128-byte line of the bf16 states: the halves written by neighbouring tiles are then merged there and
     // leave as whole lines.
     const int bh = blockIdx.x;
-    // WPB waves per block: a block is a 32x32 tile (WPB = 4) or one of its 16x16 quarters (WPB = 1)
-    const int wg = blockIdx.y * WPB + (threadIdx.x >> 6);
-    const int tile_v = (wg >> 2) / TPD, tile_k = (wg >> 2) % TPD;
-    const int lane = threadIdx.x & 63, wave = wg & 3;
+    const int tile_v = (blockIdx.y >> 2) / TPD, tile_k = (blockIdx.y >> 2) % TPD;   // 32x32 tile, then its quarter
+    const int lane = threadIdx.x, wave = blockIdx.y & 3;
     const int ti = lane >> 3, tj = lane & 7;
     const int dv0 = 32 * tile_v + 16 * (wave >> 1) + 2 * ti;
     const int dk0 = 32 * tile_k + 16 * (wave & 1) + 2 * tj;
@@ -261,14 +261,12 @@ template <typename T, int D>
 int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hin, const float *prodT,
                       const float *decay, void *statesT, void *statesN, void *hout, int tail)
 {
-    dim3 grid(BH, (D / 32) * (D / 32)), block(256);
-    if ((int64_t)grid.y * BH >= 256) {
+    dim3 grid(BH, (D / 16) * (D / 16)), block(64);
+    if ((int64_t)grid.y * BH >= 1024) {      // at least a wave per SIMD
         hipLaunchKernelGGL((chunk_scan_kernel<T, D, 4>), grid, block, 0, st, (const T *)hin, prodT, decay,
                            (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
     } else {
-        // few (b,h) pairs: one wave per block, so that the quarters of a tile spread over four CUs
-        grid.y *= 4;
-        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 32, 1>), grid, dim3(64), 0, st, (const T *)hin, prodT, decay,
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 32>), grid, block, 0, st, (const T *)hin, prodT, decay,
                            (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
     }
     return launch_status();
