@@ -136,7 +136,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
                 kf[ks] = kN[ks];
                 st8(Vn + wrow + 32 * ks, vN[ks]);
             }
-            subblock_forward<T, D, true>(p, qf, kf, g + row, q + row, k + row, valid, rtab + w * D, Kh + wrow, true,
+            subblock_forward<T, D, true, false, D == 64>(p, qf, kf, g + row, q + row, k + row, valid, rtab + w * D, Kh + wrow, true,
                                    Kl + wrow, r, c, accD, qh);
         }
         __syncthreads();                     // tiles of this block and the published state are in place

@@ -73,6 +73,114 @@ __device__ __forceinline__ void bwd_level(float (&p8)[8], float (&s8)[8], const 
     hier_step<H>(p8, s8, upper);
 }
 
+// Hard gates are rare (a sub-block whose gate sums span 48 powers of two), and the dyadic levels need ~150
+// registers more than the one-anchor path.  Inlined, they set the register count of the whole kernel; as a
+// real call, the registers they clobber are saved and restored around the call only, on the path that takes it.
+typedef __attribute__((address_space(3))) BT *LdsBT;
+typedef __attribute__((address_space(3))) float *LdsF32;
+
+struct HardSliceDq {
+    float p8[8], dq8[8];
+};
+// One 32-feature slice of the own sub-block of sweep 1: dyadic levels (query part), e^{tau} of the slice into
+// the table row (lane r == 0), the rescaled key rows into the tiles; returns l_i and the sub-block's part of dq.
+template <int XS>
+__device__ __attribute__((noinline)) HardSliceDq hard_slice_dq(const float *gp, const BT *qp, const BT *kp, float live,
+                                                               float dd, f32x4 dAt, f32x4 dAn, LdsBT xh3, LdsBT xl3,
+                                                               int xnat, int xk4, LdsF32 rt3, LdsBT kh3, LdsBT kl3)
+{
+    typedef FragTypes<BT>::d8 D8;
+    const int lane = threadIdx.x & 63, r = lane & 15, c = lane >> 4;
+    BT *xh = (BT *)xh3, *xl = (BT *)xl3;
+    HardSliceDq out;
+    float s8[8], a[8], bq[8], dk8[8];
+    f32x8 gg = ld8(gp);
+    unpack8(ld8(qp), a);
+    unpack8(ld8(kp), bq);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        out.p8[e] = gg.v[e] * kLog2e * live;
+        s8[e] = 0.f;
+        a[e] *= live;
+        bq[e] *= live;
+        out.dq8[e] = dd * bq[e];
+    }
+    bwd_level<1, XS, true, false>(out.p8, s8, a, bq, dAt, dAn, xh, xl, xnat, xk4, r, c, out.dq8, dk8);
+    bwd_level<2, XS, true, false>(out.p8, s8, a, bq, dAt, dAn, xh, xl, xnat, xk4, r, c, out.dq8, dk8);
+    bwd_level<4, XS, true, false>(out.p8, s8, a, bq, dAt, dAn, xh, xl, xnat, xk4, r, c, out.dq8, dk8);
+    bwd_level<8, XS, true, false>(out.p8, s8, a, bq, dAt, dAn, xh, xl, xnat, xk4, r, c, out.dq8, dk8);
+    // p8 = l_i, s8 = tau - l_i
+    if (r == 0) {
+        f32x8 t;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(out.p8[e] + s8[e]);
+        st8((float *)rt3, t);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) bq[e] *= fast_exp2(s8[e]);
+    D8 kh, kl;
+    split8<BT>(bq, kh, kl);
+    st8((BT *)kh3, kh);
+    st8((BT *)kl3, kl);
+    return out;
+}
+
+struct HardSliceRev {
+    float s8[8], dk8[8], kt8[8];
+    f32x4 G[4];
+    float dot;
+};
+// The same for sweep 2: key part of the levels, the levels' scores (added to G, one block per level), q.k
+// (added to dot), e^{tau} of the slice into the table row, the rescaled query rows (head, remainder) into the tiles;
+// returns tau - l_i, the sub-block's part of dk and k e^{tau - l_i}.
+template <int XS>
+__device__ __attribute__((noinline)) HardSliceRev hard_slice_rev(const float *gp, const BT *qp, const BT *kp, float live,
+                                                                 float dd, f32x4 dAt, f32x4 dAn, f32x4 G0, f32x4 G1,
+                                                                 f32x4 G2, f32x4 G3, float dot, LdsBT xh3, LdsBT xl3,
+                                                                 int xnat, int xk4, LdsF32 rt3, LdsBT qh3, LdsBT ql3)
+{
+    typedef FragTypes<BT>::d8 D8;
+    const int lane = threadIdx.x & 63, r = lane & 15, c = lane >> 4;
+    BT *xh = (BT *)xh3, *xl = (BT *)xl3;
+    HardSliceRev out;
+    out.G[0] = G0; out.G[1] = G1; out.G[2] = G2; out.G[3] = G3;
+    out.dot = dot;
+    float p8[8], a[8], bq[8], dq8[8];
+    f32x8 gg = ld8(gp);
+    unpack8(ld8(qp), a);
+    unpack8(ld8(kp), bq);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        p8[e] = gg.v[e] * kLog2e * live;
+        out.s8[e] = 0.f;
+        a[e] *= live;
+        bq[e] *= live;
+        out.dk8[e] = dd * a[e];
+        out.dot += a[e] * bq[e];
+    }
+    bwd_level<1, XS, false, true, true>(p8, out.s8, a, bq, dAt, dAn, xh, xl, xnat, xk4, r, c, dq8, out.dk8, &out.G[0]);
+    bwd_level<2, XS, false, true, true>(p8, out.s8, a, bq, dAt, dAn, xh, xl, xnat, xk4, r, c, dq8, out.dk8, &out.G[1]);
+    bwd_level<4, XS, false, true, true>(p8, out.s8, a, bq, dAt, dAn, xh, xl, xnat, xk4, r, c, dq8, out.dk8, &out.G[2]);
+    bwd_level<8, XS, false, true, true>(p8, out.s8, a, bq, dAt, dAn, xh, xl, xnat, xk4, r, c, dq8, out.dk8, &out.G[3]);
+    if (r == 0) {
+        f32x8 t;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p8[e] + out.s8[e]);
+        st8((float *)rt3, t);
+    }
+    float qe[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        qe[e] = a[e] * fast_exp2(p8[e]);
+        out.kt8[e] = bq[e] * fast_exp2(out.s8[e]);
+    }
+    D8 h8, l8;
+    split8<BT>(qe, h8, l8);
+    st8((BT *)qh3, h8);
+    st8((BT *)ql3, l8);
+    return out;
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------------
@@ -251,42 +359,17 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
             } else {
                 // hard gates: the dyadic levels, 32 features at a time, inputs fetched again
                 const float live = valid ? 1.f : 0.f;
-#pragma unroll
+#pragma unroll 1
                 for (int ks = 0; ks < KS; ++ks) {
-                    float p8[8], s8[8], a[8], bq[8], dq8[8], dk8[8];
-                    f32x8 gg = ld8(refetch(g + row) + 32 * ks + 8 * c);
-                    unpack8(ld8(refetch(q + row) + 32 * ks + 8 * c), a);
-                    unpack8(ld8(refetch(k + row) + 32 * ks + 8 * c), bq);
+                    const HardSliceDq hs = hard_slice_dq<XS>(
+                        g + row + 32 * ks + 8 * c, q + row + 32 * ks + 8 * c, k + row + 32 * ks + 8 * c, live, dd, dAt, dAn,
+                        (LdsBT)xh, (LdsBT)xl, Lx.nat, Lx.k4, (LdsF32)(rt + 32 * ks + 8 * c), (LdsBT)(Kh + wrow + 32 * ks),
+                        (LdsBT)(Kl + wrow + 32 * ks));
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
-                        p8[e] = gg.v[e] * kLog2e * live;
-                        s8[e] = 0.f;
-                        a[e] *= live;
-                        bq[e] *= live;
-                        dq8[e] = dd * bq[e];
+                        p[8 * ks + e] = hs.p8[e];
+                        dqo[8 * ks + e] = hs.dq8[e];
                     }
-                    bwd_level<1, XS, true, false>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8);
-                    bwd_level<2, XS, true, false>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8);
-                    bwd_level<4, XS, true, false>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8);
-                    bwd_level<8, XS, true, false>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8);
-                    // p8 = l_i, s8 = tau - l_i
-                    if (r == 0) {
-                        f32x8 t;
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p8[e] + s8[e]);
-                        st8(rt + 32 * ks + 8 * c, t);
-                    }
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        p[8 * ks + e] = p8[e];
-                        dqo[8 * ks + e] = dq8[e];
-                        bq[e] *= fast_exp2(s8[e]);
-                    }
-                    D8 kh, kl;
-                    split8<T>(bq, kh, kl);
-                    st8(Kh + wrow + 32 * ks, kh);
-                    st8(Kl + wrow + 32 * ks, kl);
-                    __builtin_amdgcn_sched_barrier(0);
                 }
                 lowTh = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
                 lowTl = lowTh;
@@ -625,44 +708,21 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
             } else {
                 const float live = valid ? 1.f : 0.f;
                 f32x4 Gl[4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-#pragma unroll
+#pragma unroll 1
                 for (int ks = 0; ks < KS; ++ks) {
-                    float p8[8], s8[8], a[8], bq[8], dq8[8], dk8[8];
-                    f32x8 gg = ld8(refetch(g + row) + 32 * ks + 8 * c);
-                    unpack8(ld8(refetch(q + row) + 32 * ks + 8 * c), a);
-                    unpack8(ld8(refetch(k + row) + 32 * ks + 8 * c), bq);
+                    const HardSliceRev hs = hard_slice_rev<XS>(
+                        g + row + 32 * ks + 8 * c, q + row + 32 * ks + 8 * c, k + row + 32 * ks + 8 * c, live, dd, dAt, dAn,
+                        Gl[0], Gl[1], Gl[2], Gl[3], dot, (LdsBT)xh, (LdsBT)xl, Lx.nat, Lx.k4,
+                        (LdsF32)(rt + 32 * ks + 8 * c), (LdsBT)(Qh + wrow + 32 * ks), (LdsBT)(Ql + wrow + 32 * ks));
+#pragma unroll
+                    for (int l = 0; l < 4; ++l) Gl[l] = hs.G[l];
+                    dot = hs.dot;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
-                        p8[e] = gg.v[e] * kLog2e * live;
-                        s8[e] = 0.f;
-                        a[e] *= live;
-                        bq[e] *= live;
-                        dk8[e] = dd * a[e];
-                        dot += a[e] * bq[e];
+                        sv[8 * ks + e] = hs.s8[e];
+                        dko[8 * ks + e] = hs.dk8[e];
+                        kt[8 * ks + e] = hs.kt8[e];
                     }
-                    bwd_level<1, XS, false, true, true>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8, &Gl[0]);
-                    bwd_level<2, XS, false, true, true>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8, &Gl[1]);
-                    bwd_level<4, XS, false, true, true>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8, &Gl[2]);
-                    bwd_level<8, XS, false, true, true>(p8, s8, a, bq, dAt, dAn, xh, xl, Lx.nat, Lx.k4, r, c, dq8, dk8, &Gl[3]);
-                    if (r == 0) {
-                        f32x8 t;
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p8[e] + s8[e]);
-                        st8(rt + 32 * ks + 8 * c, t);
-                    }
-                    float qe[8];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        sv[8 * ks + e] = s8[e];
-                        dko[8 * ks + e] = dk8[e];
-                        qe[e] = a[e] * fast_exp2(p8[e]);
-                        kt[8 * ks + e] = bq[e] * fast_exp2(s8[e]);
-                    }
-                    D8 h8, l8;
-                    split8<T>(qe, h8, l8);
-                    st8(Qh + wrow + 32 * ks, h8);
-                    st8(Ql + wrow + 32 * ks, l8);
-                    __builtin_amdgcn_sched_barrier(0);
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {

@@ -51,10 +51,88 @@ template <typename T4> __device__ __forceinline__ f32x4 mma_t_split(T4 ah, T4 al
     return mma_t(ah, bh, acc);
 }
 
+// Hard gates (a sub-block whose gate sums span 48 powers of two or more) are rare, and the dyadic levels need
+// more registers than the one-anchor path.  Inlined, they count towards the registers of the whole kernel; as a
+// real call, the registers they clobber are saved and restored around the call only, on the path that takes it.
+// That pays where the kernel is not held to a register budget of its own (a budget binds the callee too, and
+// the saves then land on the common path: the 128-register output kernel of chunk_gla went from 35 to 57 us).
+struct HardSliceFwd {
+    f32x4 G[4];
+    float dot, qh8[8];
+};
+// One 32-feature slice of a hard sub-block, the loop body of the inlined form in subblock_forward: the levels'
+// scores (added to G, one block per level), q.k (added to dot), e^{tau} of the slice into the table row (lane
+// r == 0), the rescaled key rows into the tiles (LDS); returns q e^{l_i}.  The pointers are those of the lane's 8
+// features of the slice.
+template <typename T, bool PRECISE>
+__device__ __attribute__((noinline)) HardSliceFwd hard_slice_fwd(
+    const float *gp, const T *qp, const T *kp, float live, f32x4 G0, f32x4 G1, f32x4 G2, f32x4 G3, float dot,
+    __attribute__((address_space(3))) float *rt3, __attribute__((address_space(3))) T *kh3, bool write_kh,
+    __attribute__((address_space(3))) T *kl3, bool write_kl)
+{
+    typedef typename FragTypes<T>::d8 D8;
+    const int r = threadIdx.x & 15;
+    HardSliceFwd out;
+    out.G[0] = G0; out.G[1] = G1; out.G[2] = G2; out.G[3] = G3;
+    float p8[8], s8[8], a[8], bq[8];
+    {
+        f32x8 gg = ld8(gp);
+        unpack8(ld8(qp), a);
+        unpack8(ld8(kp), bq);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            p8[e] = gg.v[e] * kLog2e * live;
+            s8[e] = 0.f;
+            a[e] *= live;
+            bq[e] *= live;
+        }
+    }
+    auto level = [&](auto hc, auto lc) {
+        constexpr int h_ = decltype(hc)::value, L_ = decltype(lc)::value;
+        const bool upper = (r & h_) != 0;
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = (upper ? a[e] : bq[e]) * fast_exp2(upper ? p8[e] : s8[e]);
+        if constexpr (PRECISE) {
+            D8 Xh, Xl;
+            split8<T>(x, Xh, Xl);
+            out.G[L_] = mma_d_split(Xh, Xl, Xh, Xl, out.G[L_]);
+        } else {
+            D8 X = pack8<T>(x);
+            out.G[L_] = mma_d(X, X, out.G[L_]);
+        }
+        hier_step<h_>(p8, s8, upper);
+    };
+    level(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+    level(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
+    level(std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
+    level(std::integral_constant<int, 8>{}, std::integral_constant<int, 3>{});
+    // p8 = l_i, s8 = tau - l_i
+    if (r == 0) {
+        f32x8 t;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p8[e] + s8[e]);
+        st8((float *)rt3, t);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        dot += a[e] * bq[e];
+        out.qh8[e] = a[e] * fast_exp2(p8[e]);
+        bq[e] *= fast_exp2(s8[e]);
+    }
+    out.dot = dot;
+    D8 kh, kl;
+    split8<T>(bq, kh, kl);
+    if (write_kh) st8((T *)kh3, kh);
+    if (write_kl) st8((T *)kl3, kl);
+    return out;
+}
+
 // PRECISE: the score products take their operands as head + remainder, for callers that promise fp32
 // arithmetic on bf16 inputs; kl_row must be given then.
 // SCANNED: p already holds the inclusive prefix sums over the rows (the caller ran prefix_sum_rows).
-template <typename T, int D, bool PRECISE = false, bool SCANNED = false>
+// CALL_HARD: the hard-gate path is a call of hard_slice_fwd per slice instead of inlined code.
+template <typename T, int D, bool PRECISE = false, bool SCANNED = false, bool CALL_HARD = false>
 __device__ __forceinline__ void subblock_forward(float (&p)[D / 4],
                                                  const typename FragTypes<T>::d8 (&qf)[D / 32],
                                                  const typename FragTypes<T>::d8 (&kf)[D / 32],
@@ -136,8 +214,25 @@ __device__ __forceinline__ void subblock_forward(float (&p)[D / 4],
         f32x4 Gl[4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
         float dot = 0.f;
         const float live = valid ? 1.f : 0.f;
+        constexpr int kInlined = CALL_HARD ? 0 : KS;
+        if constexpr (CALL_HARD) {
+            typedef __attribute__((address_space(3))) T *LdsT;
+#pragma unroll 1
+            for (int ks = 0; ks < KS; ++ks) {
+                const int fo = 32 * ks + 8 * c;
+                const HardSliceFwd hs = hard_slice_fwd<T, PRECISE>(
+                    g_row + fo, q_row + fo, k_row + fo, live, Gl[0], Gl[1], Gl[2], Gl[3], dot,
+                    (__attribute__((address_space(3))) float *)(rt + fo), (LdsT)(kh_row + 32 * ks), write_kh,
+                    (LdsT)(kl_row + 32 * ks), kl_row != nullptr);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
+                for (int l = 0; l < 4; ++l) Gl[l] = hs.G[l];
+                dot = hs.dot;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qh[8 * ks + e] = hs.qh8[e];
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < kInlined; ++ks) {
             float p8[8], s8[8], a[8], bq[8];
             {
                 f32x8 gg = ld8(refetch(g_row) + 32 * ks + 8 * c);
