@@ -163,7 +163,9 @@ __device__ __forceinline__ void subblock_forward(float (&p)[D / 4],
     }
     const bool one_anchor = wave_all_below(span, kOneAnchorSpan);
 
-    if (one_anchor) {
+    // the hint keeps the register saves that the other branch needs out of this one (chunk_gla's output kernel,
+    // held to 128 registers: 35.5 -> 33 us)
+    if (__builtin_expect(one_anchor, true)) {
         float dot = 0.f;
         f32x4 G = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
