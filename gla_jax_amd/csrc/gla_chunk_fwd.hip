@@ -157,7 +157,7 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
         float o[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
-        st8(out + rowoff + fo + 8 * c, pack8<T>(o));
+        st8_once(out + rowoff + fo + 8 * c, pack8<T>(o));
         if (ks + 1 < KS) {
             __syncthreads();             // every wave is done with the staged rows
             stage_store();
