@@ -28,9 +28,12 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
-def _canon(hidden_init, log_fgate, value, key, query):
-    """Checks the reference's shape contract and returns 4-D contiguous views
-    (h0 [B,H,DK,DV], g/k/q [B,T,H,DK], v [B,T,H,DV]) plus the leading batch shape."""
+def _prep(hidden_init, log_fgate, value, key, query):
+    """Checks the reference's shape contract and returns the canonical 4-D views the kernels take
+    (h0 [B,H,DK,DV], g/k/q [B,T,H,DK], v [B,T,H,DV]; dense, gates fp32, hidden in the value dtype), the
+    leading batch shape and the dims.  Everything here is a differentiable torch op (reshape, cast, copy),
+    so autograd carries gradients back to the caller's own layouts and dtypes; for arrays that are
+    already dense and typed as the kernels want them nothing is copied."""
     for name, t in (("hidden_init", hidden_init), ("log_fgate", log_fgate), ("value", value),
                     ("key", key), ("query", query)):
         if not isinstance(t, torch.Tensor):
@@ -49,12 +52,16 @@ def _canon(hidden_init, log_fgate, value, key, query):
     if tuple(hidden_init.shape) != lead + (H, DK, DV):
         raise AssertionError(f"hidden_init shape {tuple(hidden_init.shape)} != {lead + (H, DK, DV)}")
     dt = value.dtype
-    if dt not in _DT or key.dtype != dt or query.dtype != dt or hidden_init.dtype != dt:
-        raise TypeError("hidden_init, value, key, query must share one dtype (float32 or bfloat16)")
+    if dt not in _DT or key.dtype != dt or query.dtype != dt:
+        raise TypeError("value, key, query must share one dtype (float32 or bfloat16)")
+    if not hidden_init.dtype.is_floating_point:
+        raise TypeError("hidden_init must be a floating-point tensor")
     B = 1
     for s in lead:
         B *= s
-    h0 = hidden_init.reshape(B, H, DK, DV).contiguous()
+    # the state enters the kernels in the value dtype (the reference's chunk path casts it the same way,
+    # gla.py:720) and hidden_final goes back out in hidden_init's own dtype (gla.py:46, 727)
+    h0 = hidden_init.reshape(B, H, DK, DV).to(dt).contiguous()
     g = log_fgate.reshape(B, T, H, DK).to(torch.float32).contiguous()      # gates are fp32 (gla.py:495)
     v = value.reshape(B, T, H, DV).contiguous()
     k = key.reshape(B, T, H, DK).contiguous()
@@ -62,39 +69,45 @@ def _canon(hidden_init, log_fgate, value, key, query):
     return (h0, g, v, k, q), lead, (B, T, H, DK, DV)
 
 
-def _batched_vmap(fn_apply, n_tensor_args):
-    """vmap rule shared by the Functions below: every tensor argument already accepts leading batch
-    axes, so a vmapped call is the same call with the mapped axis moved to the front."""
-    def rule(info, in_dims, *args):
-        moved = []
-        for a, d in zip(args[:n_tensor_args], in_dims[:n_tensor_args]):
-            if d is None:
-                a = a.unsqueeze(0).expand(info.batch_size, *a.shape)
-            else:
-                a = a.movedim(d, 0)
-            moved.append(a)
-        outs = fn_apply(*moved, *args[n_tensor_args:])
-        return outs, tuple(0 for _ in outs)
-    return rule
+def _merge_mapped(info, in_dims, tensors):
+    """vmap rule helper: every Function below takes canonical arrays with ONE batch axis in front, so a mapped
+    call is the same call with the mapped axis folded into that batch axis.  Unmapped arguments are
+    broadcast.  Flat byte buffers (the residual of chunk_gla) carry no axis of their own and pass through."""
+    out = []
+    for a, d in zip(tensors, in_dims):
+        if a.dtype == torch.uint8:
+            out.append(a)
+            continue
+        a = a.unsqueeze(0).expand(info.batch_size, *a.shape) if d is None else a.movedim(d, 0)
+        out.append(a.reshape((a.shape[0] * a.shape[1],) + tuple(a.shape[2:])))
+    return out
+
+
+def _split_mapped(info, outs):
+    return tuple(o if o.dtype == torch.uint8 else o.reshape((info.batch_size, -1) + tuple(o.shape[1:]))
+                 for o in outs)
+
+
+def _no_double_backward(name):
+    raise NotImplementedError(f"{name}: second-order gradients are not provided "
+                              "(the reference defines first-order custom_vjp rules only)")
 
 
 # ------------------------------------------------------------------------------------------------
 # chunk_gla
 # ------------------------------------------------------------------------------------------------
 class _ChunkGLA(torch.autograd.Function):
-    """forward = chunk_gla_forward (gla.py:483-550); backward = chunk_gla_backward (gla.py:552-625)."""
+    """forward = chunk_gla_forward (gla.py:483-550); backward = chunk_gla_backward (gla.py:552-625).
+    Arguments are the canonical arrays of `_prep`."""
 
     @staticmethod
-    def forward(hidden_init, log_fgate, value, key, query, chunk_size):
-        (h0, g, v, k, q), lead, (B, T, H, DK, DV) = _canon(hidden_init, log_fgate, value, key, query)
+    def forward(h0, g, v, k, q, chunk_size):
+        # the kernels take dense arrays by address; a transform may hand over views (a broadcast hidden_init)
+        h0, g, v, k, q = (t.contiguous() for t in (h0, g, v, k, q))
+        B, T, H, DK = k.shape
+        DV = v.shape[-1]
         lib = _lib.load()
         dt = _DT[v.dtype]
-        if DK != DV:
-            raise AssertionError("chunk_gla needs key and value head dims to be equal")   # gla.py:499
-        if chunk_size <= 0 or chunk_size & (chunk_size - 1):
-            raise AssertionError(f"Chunk length must be power of 2, but got {chunk_size}")  # gla.py:500
-        if T % chunk_size:
-            raise AssertionError(f"sequence length {T} is not a multiple of chunk_size {chunk_size}")
         ws_bytes = lib.gla_chunk_fwd_workspace_bytes(B, T, H, DK, DV, chunk_size, dt)
         st_bytes = lib.gla_chunk_states_bytes(B, T, H, DK, DV, chunk_size, dt)
         if ws_bytes == 0 or st_bytes == 0:
@@ -106,17 +119,14 @@ class _ChunkGLA(torch.autograd.Function):
         rc = lib.gla_chunk_fwd(_stream(), B, T, H, DK, DV, chunk_size, dt, _ptr(h0), _ptr(g), _ptr(v),
                                _ptr(k), _ptr(q), _ptr(hT), _ptr(out), _ptr(states), _ptr(ws), ws_bytes)
         _lib.check("gla_chunk_fwd", rc)
-        return hT.reshape(lead + (H, DK, DV)), out.reshape(lead + (T, H, DV)), states
+        return hT, out, states
 
     @staticmethod
     def setup_context(ctx, inputs, output):
-        hidden_init, log_fgate, value, key, query, chunk_size = inputs
+        h0, g, v, k, q, chunk_size = inputs
         states = output[2]
-        (_, g, v, k, q), lead, _ = _canon(hidden_init, log_fgate, value, key, query)
-        ctx.save_for_backward(states, g, v, k, q)
+        ctx.save_for_backward(states, g, v, k, q)          # residuals of gla.py:542-549
         ctx.chunk_size = chunk_size
-        ctx.lead = lead
-        ctx.g_dtype = log_fgate.dtype
         ctx.mark_non_differentiable(states)
 
     @staticmethod
@@ -124,30 +134,53 @@ class _ChunkGLA(torch.autograd.Function):
         states, g, v, k, q = ctx.saved_tensors
         B, T, H, DK = k.shape
         DV = v.shape[-1]
+        dhT = torch.zeros(B, H, DK, DV, dtype=v.dtype, device=v.device) if dhT is None else dhT
+        dout = torch.zeros_like(v) if dout is None else dout
+        return _ChunkGLABwd.apply(states, g, v, k, q, dhT, dout, ctx.chunk_size) + (None,)
+
+    @staticmethod
+    def vmap(info, in_dims, *args):
+        outs = _ChunkGLA.apply(*_merge_mapped(info, in_dims[:5], args[:5]), args[5])
+        # the residual is one flat buffer over the merged batch; it carries no mapped axis of its own
+        return _split_mapped(info, outs), (0, 0, None)
+
+
+class _ChunkGLABwd(torch.autograd.Function):
+    """The backward rule as a function of its own, so that function transforms (torch.func.grad, vmap of a
+    gradient) reach the kernels with plain tensors."""
+
+    @staticmethod
+    def forward(states, g, v, k, q, dhT, dout, chunk_size):
+        states, g, v, k, q = (t.contiguous() for t in (states, g, v, k, q))
+        B, T, H, DK = k.shape
+        DV = v.shape[-1]
         lib = _lib.load()
         dt = _DT[v.dtype]
-        dhT = (torch.zeros(B, H, DK, DV, dtype=v.dtype, device=v.device) if dhT is None
-               else dhT.reshape(B, H, DK, DV).to(v.dtype).contiguous())
-        dout = (torch.zeros_like(v) if dout is None else dout.reshape(B, T, H, DV).to(v.dtype).contiguous())
-        ws_bytes = lib.gla_chunk_bwd_workspace_bytes(B, T, H, DK, DV, ctx.chunk_size, dt)
+        dhT = dhT.to(v.dtype).contiguous()
+        dout = dout.to(v.dtype).contiguous()
+        ws_bytes = lib.gla_chunk_bwd_workspace_bytes(B, T, H, DK, DV, chunk_size, dt)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=v.device)
         dh0 = torch.empty_like(dhT)
         dg = torch.empty_like(g)
         dv, dk, dq = torch.empty_like(v), torch.empty_like(k), torch.empty_like(q)
-        rc = lib.gla_chunk_bwd(_stream(), B, T, H, DK, DV, ctx.chunk_size, dt, _ptr(g), _ptr(v), _ptr(k),
+        rc = lib.gla_chunk_bwd(_stream(), B, T, H, DK, DV, chunk_size, dt, _ptr(g), _ptr(v), _ptr(k),
                                _ptr(q), _ptr(states), _ptr(dhT), _ptr(dout), _ptr(dh0), _ptr(dg),
                                _ptr(dv), _ptr(dk), _ptr(dq), _ptr(ws), ws_bytes)
         _lib.check("gla_chunk_bwd", rc)
-        lead = ctx.lead
-        return (dh0.reshape(lead + (H, DK, DV)), dg.reshape(lead + (T, H, DK)).to(ctx.g_dtype),
-                dv.reshape(lead + (T, H, DV)), dk.reshape(lead + (T, H, DK)),
-                dq.reshape(lead + (T, H, DK)), None)
+        return dh0, dg, dv, dk, dq
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        pass
+
+    @staticmethod
+    def backward(ctx, *grads):
+        _no_double_backward("chunk_gla")
 
     @staticmethod
     def vmap(info, in_dims, *args):
-        outs, dims = _batched_vmap(_ChunkGLA.apply, 5)(info, in_dims, *args)
-        # the residual is flattened over the batch; it carries no mapped axis of its own
-        return outs, (0, 0, None)
+        outs = _ChunkGLABwd.apply(*_merge_mapped(info, in_dims[:7], args[:7]), args[7])
+        return _split_mapped(info, outs), (0,) * 5
 
 
 def chunk_gla(hidden_init, log_fgate, value, key, query, chunk_size, block_size_t: int = 64,
@@ -161,8 +194,16 @@ def chunk_gla(hidden_init, log_fgate, value, key, query, chunk_size, block_size_
     and have no effect here.  Differentiable in all five array arguments (gla.py:625)."""
     if interpret:
         raise ValueError("interpret=True asks for the reference's CPU interpreter; this build has no CPU path")
-    hT, out = _ChunkGLA.apply(hidden_init, log_fgate, value, key, query, int(chunk_size))[:2]
-    return hT, out
+    chunk_size = int(chunk_size)
+    (h0, g, v, k, q), lead, (B, T, H, DK, DV) = _prep(hidden_init, log_fgate, value, key, query)
+    if DK != DV:
+        raise AssertionError("chunk_gla needs key and value head dims to be equal")   # gla.py:499
+    if chunk_size <= 0 or chunk_size & (chunk_size - 1):
+        raise AssertionError(f"Chunk length must be power of 2, but got {chunk_size}")  # gla.py:500
+    if T % chunk_size:
+        raise AssertionError(f"sequence length {T} is not a multiple of chunk_size {chunk_size}")
+    hT, out = _ChunkGLA.apply(h0, g, v, k, q, chunk_size)[:2]
+    return hT.reshape(lead + (H, DK, DV)).to(hidden_init.dtype), out.reshape(lead + (T, H, DV))
 
 
 # ------------------------------------------------------------------------------------------------
@@ -170,13 +211,14 @@ def chunk_gla(hidden_init, log_fgate, value, key, query, chunk_size, block_size_
 # ------------------------------------------------------------------------------------------------
 class _RecurrentGLA(torch.autograd.Function):
     """forward = recurrent_gla_forward (gla.py:99-170); backward = recurrent_gla_backward
-    (gla.py:172-269).  `out_fp32` selects the fp32 output of the naive flavour (gla.py:37)."""
+    (gla.py:172-269).  `out_fp32` selects the fp32 output of the naive flavour (gla.py:37).
+    Arguments are the canonical arrays of `_prep`."""
 
     @staticmethod
-    def forward(hidden_init, log_fgate, value, key, query, reverse, out_fp32):
-        (h0, g, v, k, q), lead, (B, T, H, DK, DV) = _canon(hidden_init, log_fgate, value, key, query)
-        if DK != DV:
-            raise AssertionError("Not supported yet: key and value head dims differ")      # gla.py:120, 391
+    def forward(h0, g, v, k, q, reverse, out_fp32):
+        h0, g, v, k, q = (t.contiguous() for t in (h0, g, v, k, q))
+        B, T, H, DK = k.shape
+        DV = v.shape[-1]
         lib = _lib.load()
         dt = _DT[v.dtype]
         odt = _lib.GLA_F32 if out_fp32 else dt
@@ -185,48 +227,72 @@ class _RecurrentGLA(torch.autograd.Function):
         rc = lib.gla_recurrent_fwd(_stream(), B, T, H, DK, DV, dt, odt, int(bool(reverse)), _ptr(h0),
                                    _ptr(g), _ptr(v), _ptr(k), _ptr(q), _ptr(hT), _ptr(out))
         _lib.check("gla_recurrent_fwd", rc)
-        return hT.reshape(lead + (H, DK, DV)), out.reshape(lead + (T, H, DV))
+        return hT, out
 
     @staticmethod
     def setup_context(ctx, inputs, output):
-        hidden_init, log_fgate, value, key, query, reverse, out_fp32 = inputs
-        hT = output[0]
-        (h0, g, v, k, q), lead, _ = _canon(hidden_init, log_fgate, value, key, query)
-        ctx.save_for_backward(h0, g, v, k, q, hT)          # residuals of gla.py:169
+        h0, g, v, k, q, reverse, out_fp32 = inputs
+        ctx.save_for_backward(h0, g, v, k, q, output[0])          # residuals of gla.py:169
         ctx.reverse = bool(reverse)
         ctx.out_fp32 = bool(out_fp32)
-        ctx.lead = lead
-        ctx.g_dtype = log_fgate.dtype
 
     @staticmethod
     def backward(ctx, dhT, dout):
         h0, g, v, k, q, hT = ctx.saved_tensors
+        o_torch = torch.float32 if ctx.out_fp32 else v.dtype
+        dhT = torch.zeros_like(h0) if dhT is None else dhT
+        dout = torch.zeros(v.shape, dtype=o_torch, device=v.device) if dout is None else dout
+        return _RecurrentGLABwd.apply(h0, g, v, k, q, hT, dhT, dout, ctx.reverse, ctx.out_fp32) + (None, None)
+
+    @staticmethod
+    def vmap(info, in_dims, *args):
+        outs = _RecurrentGLA.apply(*_merge_mapped(info, in_dims[:5], args[:5]), args[5], args[6])
+        return _split_mapped(info, outs), (0, 0)
+
+
+class _RecurrentGLABwd(torch.autograd.Function):
+    """The backward rule of recurrent_gla as a function of its own (see _ChunkGLABwd)."""
+
+    @staticmethod
+    def forward(h0, g, v, k, q, hT, dhT, dout, reverse, out_fp32):
+        h0, g, v, k, q = (t.contiguous() for t in (h0, g, v, k, q))
         B, T, H, DK = k.shape
         DV = v.shape[-1]
         lib = _lib.load()
         dt = _DT[v.dtype]
-        odt = _lib.GLA_F32 if ctx.out_fp32 else dt
-        o_torch = torch.float32 if ctx.out_fp32 else v.dtype
-        dhT = (torch.zeros_like(h0) if dhT is None else dhT.reshape(B, H, DK, DV).to(v.dtype).contiguous())
-        dout = (torch.zeros(v.shape, dtype=o_torch, device=v.device) if dout is None
-                else dout.reshape(B, T, H, DV).to(o_torch).contiguous())
-        hTc = hT.reshape(B, H, DK, DV).contiguous()
+        odt = _lib.GLA_F32 if out_fp32 else dt
+        dhT = dhT.to(v.dtype).contiguous()
+        dout = dout.to(torch.float32 if out_fp32 else v.dtype).contiguous()
+        hTc = hT.contiguous()
         dh0 = torch.empty_like(h0)
         dg = torch.empty_like(g)
         dv, dk, dq = torch.empty_like(v), torch.empty_like(k), torch.empty_like(q)
-        rc = lib.gla_recurrent_bwd(_stream(), B, T, H, DK, DV, dt, odt, int(ctx.reverse), _ptr(h0), _ptr(g),
+        rc = lib.gla_recurrent_bwd(_stream(), B, T, H, DK, DV, dt, odt, int(bool(reverse)), _ptr(h0), _ptr(g),
                                    _ptr(v), _ptr(k), _ptr(q), _ptr(hTc), _ptr(dhT), _ptr(dout),
                                    _ptr(dh0), _ptr(dg), _ptr(dv), _ptr(dk), _ptr(dq))
         _lib.check("gla_recurrent_bwd", rc)
-        lead = ctx.lead
-        return (dh0.reshape(lead + (H, DK, DV)), dg.reshape(lead + (T, H, DK)).to(ctx.g_dtype),
-                dv.reshape(lead + (T, H, DV)), dk.reshape(lead + (T, H, DK)),
-                dq.reshape(lead + (T, H, DK)), None, None)
+        return dh0, dg, dv, dk, dq
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        pass
+
+    @staticmethod
+    def backward(ctx, *grads):
+        _no_double_backward("recurrent_gla")
 
     @staticmethod
     def vmap(info, in_dims, *args):
-        outs, dims = _batched_vmap(_RecurrentGLA.apply, 5)(info, in_dims, *args)
-        return outs, (0, 0)
+        outs = _RecurrentGLABwd.apply(*_merge_mapped(info, in_dims[:8], args[:8]), args[8], args[9])
+        return _split_mapped(info, outs), (0,) * 5
+
+
+def _recurrent(hidden_init, log_fgate, value, key, query, reverse, out_fp32):
+    (h0, g, v, k, q), lead, (B, T, H, DK, DV) = _prep(hidden_init, log_fgate, value, key, query)
+    if DK != DV:
+        raise AssertionError("Not supported yet: key and value head dims differ")      # gla.py:120, 391
+    hT, out = _RecurrentGLA.apply(h0, g, v, k, q, bool(reverse), bool(out_fp32))
+    return hT.reshape(lead + (H, DK, DV)).to(hidden_init.dtype), out.reshape(lead + (T, H, DV))
 
 
 def recurrent_gla(hidden_init, log_fgate, value, key, query, reverse: bool = False,
@@ -237,8 +303,7 @@ def recurrent_gla(hidden_init, log_fgate, value, key, query, reverse: bool = Fal
     `num_warps`, `num_stages`, `interpret` are the reference's Triton knobs: accepted, no effect."""
     if interpret:
         raise ValueError("interpret=True asks for the reference's CPU interpreter; this build has no CPU path")
-    hT, out = _RecurrentGLA.apply(hidden_init, log_fgate, value, key, query, bool(reverse), False)[:2]
-    return hT, out
+    return _recurrent(hidden_init, log_fgate, value, key, query, reverse, False)
 
 
 def recurrent_gla_naive(hidden, log_fgate, value, key, query, reverse):
@@ -246,5 +311,4 @@ def recurrent_gla_naive(hidden, log_fgate, value, key, query, reverse):
     state.  `out` comes back in float32 (promotion at gla.py:37), `hidden` in its input dtype
     (gla.py:46).  On this build it runs the same per-timestep HIP kernel as `recurrent_gla`, writing
     fp32 outputs."""
-    hT, out = _RecurrentGLA.apply(hidden, log_fgate, value, key, query, bool(reverse), True)[:2]
-    return hT, out
+    return _recurrent(hidden, log_fgate, value, key, query, reverse, True)

@@ -287,26 +287,30 @@ def _intra_forward(lam, v, k, q, block_size_t, rnd, dtype):
 
 def _intra_backward(lam, v, k, q, dout, scores, block_size_t, rnd, dtype):
     """compute_intra_contrib_backward (gla.py:857-960).  Saved scores are reused (popped, outermost
-    level first).  Returns (dlam, dv, dk, dq)."""
+    level first).  `rnd` marks what the reference stores in the input dtype: dvalue and dscore are plain
+    matmuls of bf16 operands, whose result takes the operand dtype (gla.py:880-881, 926-927); dkey and
+    dquery leave the score kernel and attention_backward in the key/query dtype (gla.py:1185-1186, 893, 900)
+    and are summed in it (gla.py:953-955); d(log_lambda) and the products feeding it stay fp32
+    (matmul_fp32, gla.py:892-901, 1073-1087).  Returns (dlam, dv, dk, dq)."""
     scores = list(scores)
 
     def rec(lam, v, k, q, do):
         N, C, D = lam.shape
         sc = scores.pop()
         if C <= block_size_t:
-            dv = np.swapaxes(sc, -1, -2) @ do                    # gla.py:926
-            dsc = do @ np.swapaxes(v, -1, -2)                    # gla.py:927
+            dv = rnd(np.swapaxes(sc, -1, -2) @ do).astype(dtype)          # gla.py:926
+            dsc = rnd(do @ np.swapaxes(v, -1, -2)).astype(dtype)          # gla.py:927
             outs = [compute_score_backward(lam[n], k[n], q[n], dsc[n], rnd, dtype) for n in range(N)]
             dlam = np.stack([o[0] for o in outs])
-            dk = np.stack([o[1] for o in outs])
-            dq = np.stack([o[2] for o in outs])
+            dk = rnd(np.stack([o[1] for o in outs])).astype(dtype)        # gla.py:1185
+            dq = rnd(np.stack([o[2] for o in outs])).astype(dtype)        # gla.py:1186
             return dlam, dv, dk, dq
         M = C // 2
         halves = [a.reshape(2 * N, M, D) for a in (lam, v, k, q, do)]
         dlam, dv, dk, dq = (a.reshape(N, C, D) for a in rec(*halves))
         # attention_backward, gla.py:878-906
-        dv_i = np.swapaxes(sc, -1, -2) @ do[:, M:]
-        dsc = do[:, M:] @ np.swapaxes(v[:, :M], -1, -2)
+        dv_i = rnd(np.swapaxes(sc, -1, -2) @ do[:, M:]).astype(dtype)
+        dsc = rnd(do[:, M:] @ np.swapaxes(v[:, :M], -1, -2)).astype(dtype)
         anchor = lam[:, M - 1:M]
         wq = np.exp(lam[:, M:] - anchor)
         wk = np.exp(anchor - lam[:, :M])
@@ -315,11 +319,11 @@ def _intra_backward(lam, v, k, q, dout, scores, block_size_t, rnd, dtype):
         dqw = dsc @ kw
         dkw = np.swapaxes(dsc, -1, -2) @ qw
         dlam = dlam.copy(); dv = dv.copy(); dk = dk.copy(); dq = dq.copy()
-        dq[:, M:] += dqw * wq
-        dk[:, :M] += dkw * wk
+        dq[:, M:] = rnd(dq[:, M:] + rnd(dqw * wq)).astype(dtype)         # gla.py:893, 954
+        dk[:, :M] = rnd(dk[:, :M] + rnd(dkw * wk)).astype(dtype)         # gla.py:900, 955
         dlam[:, M:] += dqw * qw
         dlam[:, :M] -= dkw * kw
-        dv[:, :M] += dv_i
+        dv[:, :M] = rnd(dv[:, :M] + dv_i).astype(dtype)                  # gla.py:953
         return dlam, dv, dk, dq
 
     return rec(lam, v, k, q, dout)
@@ -344,7 +348,10 @@ def _chunk_head_forward(h0, g, v, k, q, block_size_t, rnd, dtype):
 
 
 def _chunk_head_backward(g, v, k, q, res, dhidden_final, dout, block_size_t, rnd, dtype):
-    """chunk_gla_backward for one head (gla.py:552-625, 731-790)."""
+    """chunk_gla_backward for one head (gla.py:552-625, 731-790).  `rnd` marks what the reference holds in
+    the input dtype: dstate = Q~^T dO and dvalue = K~ dkv are plain matmuls of bf16 operands (gla.py:750,
+    775), the reverse scan returns its states in the dtype of dstate (ops.py:326, 373-374), dquery is cast
+    (gla.py:753); dkey of this path stays fp32 (gla.py:778), as does everything that feeds d(log_fgate)."""
     scores, state = res
     lam = cumsum(g, axis=-2, dtype=dtype)
     lam_chunk = lam[:, -1, :]
@@ -352,23 +359,25 @@ def _chunk_head_backward(g, v, k, q, res, dhidden_final, dout, block_size_t, rnd
     # compute_inter_contrib_backward, gla.py:731-790
     log_gamma = lam_chunk[:, None, :] - lam
     qw = rnd(q * np.exp(lam)).astype(dtype)
-    dstate = np.swapaxes(qw, -1, -2) @ dout                       # gla.py:750
+    dstate = rnd(np.swapaxes(qw, -1, -2) @ dout).astype(dtype)    # gla.py:750
     dqw = dout @ np.swapaxes(state, -1, -2)                       # gla.py:752
-    dq_o = dqw * np.exp(lam)
+    dq_o = rnd(dqw * np.exp(lam)).astype(dtype)                   # gla.py:753
     dlam_q = dqw * qw
     _, dkv = rnn_scan(lam_chunk, dstate, np.zeros_like(lam_chunk[0]), dhidden_final,
                       reverse=True, dtype=dtype)                  # gla.py:759-765
+    dkv = rnd(dkv).astype(dtype)                                   # ops.py:326, 373-374
     allst = np.concatenate([dkv, np.asarray(dhidden_final, dtype=dtype)[None]], axis=0)
     dh0, dkv = allst[0], allst[1:]                                 # gla.py:768-771
     kw = rnd(k * np.exp(log_gamma)).astype(dtype)
-    dv_o = kw @ dkv
+    dv_o = rnd(kw @ dkv).astype(dtype)                             # gla.py:775
     dkw = v @ np.swapaxes(dkv, -1, -2)
     dk_o = dkw * np.exp(log_gamma)
     dlam_k = -dkw * kw
     dlam_chunk = -dlam_k.sum(axis=1) + (state * np.exp(lam_chunk)[:, :, None] * dkv).sum(axis=-1)
     dlam = dlam_k + dlam_q + dlam_i                                # gla.py:786, 615
     dg = cumsum(dlam, axis=-2, init=dlam_chunk, reverse=True, dtype=dtype)   # gla.py:616-617
-    return dh0, dg, dv_o + dv_i, dk_o + dk_i, dq_o + dq_i
+    return (dh0, dg, rnd(dv_o + dv_i).astype(dtype), dk_o + dk_i,
+            rnd(dq_o + dq_i).astype(dtype))                        # gla.py:618-620
 
 
 def _to_heads(x, chunk_size):

@@ -1,13 +1,15 @@
 """GPU parity of chunk_gla (forward and all five gradients) through the C ABI against the oracle's
-naive recurrence.  Tolerance (north_star): max|err| / RMS(oracle) <= 2e-2 for bf16, <= 1e-4 for fp32
-(plus the storage rounding of bf16 outputs, see tests/util.py)."""
+naive recurrence.  Tolerance (north_star): max|err| / RMS(oracle) <= 2e-2 for bf16, <= 1e-4 for fp32; for
+bf16 the bound widens to 1.5 x the error of the emulated reference on the same inputs where that is
+larger (tests/util.py)."""
 import numpy as np
 import pytest
 import torch
 
 from oracle import gla_oracle as O
 from oracle import naive_c
-from tests.util import TOL, assert_close, cotangents, gpu_inputs, grad_kinds, to_dev, to_np
+from tests.util import (GRAD_NAMES, TOL, assert_parity, assert_plain, check_chunk_outputs, cotangents, fmt_log,
+                        gpu_inputs, loss_of, reference_emulation, to_dev, to_np)
 
 pytestmark = pytest.mark.gpu
 
@@ -37,9 +39,7 @@ def test_chunk_forward_matches_oracle(dtype, B, T, H, D, chunk, shift):
     (h0, g, v, k, q), dev = gpu_inputs(B, T, H, D, shift, seed=T + D + chunk, dtype=dtype)
     hT, out = chunk_gla(*dev, chunk)
     assert out.dtype == dtype and hT.dtype == dtype and out.shape == dev[2].shape
-    eh, eo = O.recurrent_gla_naive(h0, g, v, k, q)
-    assert_close("out", to_np(out), eo, TOL[dtype], stored=dtype)
-    assert_close("hidden_final", to_np(hT), eh, TOL[dtype], stored=dtype)
+    print(fmt_log(check_chunk_outputs(dtype, (h0, g, v, k, q), chunk, hT, out)))
 
 
 @pytest.mark.parametrize("dtype,B,T,H,D,chunk,shift", CASES)
@@ -49,12 +49,8 @@ def test_chunk_backward_matches_oracle(dtype, B, T, H, D, chunk, shift):
     dhT, dout = cotangents(h0, v, 5, dtype)
     dev = [t.clone().requires_grad_(True) for t in dev]
     hT, out = chunk_gla(*dev, chunk)
-    loss = (hT.float() * to_dev(dhT, torch.float32)).sum() + (out.float() * to_dev(dout, torch.float32)).sum()
-    grads = torch.autograd.grad(loss, dev)
-    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout)
-    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                grad_kinds(dtype)):
-        assert_close(name, to_np(got), e, TOL[dtype], stored=st)
+    grads = torch.autograd.grad(loss_of(hT, out, dhT, dout), dev)
+    print(fmt_log(check_chunk_outputs(dtype, (h0, g, v, k, q), chunk, hT, out, grads, dhT, dout)))
 
 
 def test_chunk_strong_decay_and_hard_resets():
@@ -68,9 +64,7 @@ def test_chunk_strong_decay_and_hard_resets():
     g[:, 100:104] = -90.0
     dev[1] = to_dev(g, torch.float32)
     hT, out = chunk_gla(*dev, 128)
-    eh, eo = O.recurrent_gla_naive(h0, g, v, k, q)
-    assert_close("out", to_np(out), eo, TOL[dtype], stored=dtype)
-    assert_close("hidden_final", to_np(hT), eh, TOL[dtype], stored=dtype)
+    print(fmt_log(check_chunk_outputs(dtype, (h0, g, v, k, q), 128, hT, out)))
 
 
 def test_chunk_fp32_closed_gates_do_not_cost_precision():
@@ -86,8 +80,8 @@ def test_chunk_fp32_closed_gates_do_not_cost_precision():
     eh, eo = O.recurrent_gla_naive(h0, g, v, k, q)
     for chunk in (32, 64):
         hT, out = chunk_gla(*dev, chunk)
-        assert_close("out", to_np(out), eo, 2e-5, stored=dtype)
-        assert_close("hidden_final", to_np(hT), eh, 2e-5, stored=dtype)
+        assert_plain("out", to_np(out), eo, 2e-5)
+        assert_plain("hidden_final", to_np(hT), eh, 2e-5)
 
 
 @pytest.mark.parametrize("regime", ["mild", "mixed", "resets"])
@@ -106,15 +100,8 @@ def test_chunk_backward_over_gate_regimes(regime):
     dhT, dout = cotangents(h0, v, 6, dtype)
     dev = [t.clone().requires_grad_(True) for t in dev]
     hT, out = chunk_gla(*dev, 128)
-    eh, eo = O.recurrent_gla_naive(h0, g, v, k, q)
-    assert_close("out", to_np(out), eo, TOL[dtype], stored=dtype)
-    assert_close("hidden_final", to_np(hT), eh, TOL[dtype], stored=dtype)
-    loss = (hT.float() * to_dev(dhT, torch.float32)).sum() + (out.float() * to_dev(dout, torch.float32)).sum()
-    grads = torch.autograd.grad(loss, dev)
-    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout)
-    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                grad_kinds(dtype)):
-        assert_close(name, to_np(got), e, TOL[dtype], stored=st)
+    grads = torch.autograd.grad(loss_of(hT, out, dhT, dout), dev)
+    print(fmt_log(check_chunk_outputs(dtype, (h0, g, v, k, q), 128, hT, out, grads, dhT, dout)))
 
 
 def test_chunk_size_and_concatenation_invariance():
@@ -143,38 +130,74 @@ def test_chunk_rejects_what_the_reference_rejects():
         chunk_gla(*dev, 8)                  # below the smallest tile built here
 
 
-def _full_shape_check(B, T, H, D, chunk, shift, seed, heads):
-    """Forward + all gradients at a BASELINE shape against the C restatement of the naive recurrence
-    (fp64) on the listed heads (all batches)."""
+def _full_shape_check(B, T, H, D, chunk, shift, seed, plain=()):
+    """Forward + all gradients at a BASELINE shape, EVERY batch entry and head, against the C restatement of
+    the naive recurrence (fp64) and the emulated reference on the same inputs."""
     from gla_jax_amd import chunk_gla
     dtype = torch.bfloat16
     (h0, g, v, k, q), dev = gpu_inputs(B, T, H, D, shift, seed=seed, dtype=dtype)
     dhT, dout = cotangents(h0, v, seed, dtype)
     dev = [t.clone().requires_grad_(True) for t in dev]
     hT, out = chunk_gla(*dev, chunk)
-    loss = (hT.float() * to_dev(dhT, torch.float32)).sum() + (out.float() * to_dev(dout, torch.float32)).sum()
-    grads = torch.autograd.grad(loss, dev)
-    hs = list(heads)
-    sl = lambda a: np.ascontiguousarray(a[:, :, hs]) if a.ndim == 4 and a.shape[1] == T else np.ascontiguousarray(a[:, hs])
-    exp = naive_c.naive_bwd(sl(h0), sl(g), sl(v), sl(k), sl(q), sl(dhT), sl(dout), dtype=np.float64, nthreads=16)
-    raw = {}
-    raw["out"] = assert_close("out", sl(to_np(out)), exp[6], TOL[dtype], stored=dtype)
-    raw["hidden_final"] = assert_close("hidden_final", sl(to_np(hT)), exp[5], TOL[dtype], stored=dtype)
-    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                grad_kinds(dtype)):
-        raw[name] = assert_close(name, sl(to_np(got)), e, TOL[dtype], stored=st)
-    print("plain max|err|/rms:", {k_: f"{v_:.2e}" for k_, v_ in raw.items()})
-    return raw
+    grads = torch.autograd.grad(loss_of(hT, out, dhT, dout), dev)
+    exact = naive_c.naive_bwd(h0, g, v, k, q, dhT, dout, dtype=np.float64, nthreads=16)
+    log = check_chunk_outputs(dtype, (h0, g, v, k, q), chunk, hT, out, grads, dhT, dout, exact=exact, plain=plain)
+    print("max|err|/rms:", fmt_log(log))
+    return log, dev, (hT, out) + tuple(grads), (dhT, dout)
 
 
 def test_chunk_baseline_config_fwd_bwd_full_shape():
-    """BASELINE configs[1]/[2]: B4,T4096,H6,D128, chunk 128, gates log_sigmoid(5+N(0,1)); every head."""
-    raw = _full_shape_check(4, 4096, 6, 128, 128, 5.0, seed=12, heads=range(6))
-    # weak decay: the plain north_star metric (no allowance) stays at the 2e-2 level for every output
-    assert max(raw.values()) <= 3e-2
+    """BASELINE configs[1]/[2]: B4,T4096,H6,D128, chunk 128, gates log_sigmoid(5+N(0,1)).  Under weak decay the
+    final state and the gradient of the initial one meet the plain north_star bound (no allowance)."""
+    log, _, _, _ = _full_shape_check(4, 4096, 6, 128, 128, 5.0, seed=12, plain=("hidden_final", "dhidden_init"))
+    assert max(a for a, _ in log.values()) <= 3e-2
 
 
 def test_chunk_long_context_strong_decay_full_shape():
-    """BASELINE configs[3]: B1,T32768,H8,D128, chunk 128, gates log_sigmoid(N(0,1)); heads 0 and 5 are
-    checked against the oracle (the other six run the same kernels on other data)."""
-    _full_shape_check(1, 32768, 8, 128, 128, 0.0, seed=13, heads=(0, 5))
+    """BASELINE configs[3]: B1,T32768,H8,D128, chunk 128, gates log_sigmoid(N(0,1)): all eight heads against
+    the oracle, and every head run alone equals, bit for bit, the same head of the full run."""
+    from gla_jax_amd import chunk_gla
+    log, dev, full, (dhT, dout) = _full_shape_check(1, 32768, 8, 128, 128, 0.0, seed=13)
+    for h in (0, 3, 7):
+        one = [(t.detach()[:, h:h + 1] if i == 0 else t.detach()[:, :, h:h + 1]).contiguous().requires_grad_(True)
+               for i, t in enumerate(dev)]          # dev[0] is hidden_init [B,H,D,D], the rest are [B,T,H,D]
+        hT1, out1 = chunk_gla(*one, 128)
+        g1 = torch.autograd.grad(loss_of(hT1, out1, dhT[:, h:h + 1], dout[:, :, h:h + 1]), one)
+        for name, a, b in zip(("hidden_final", "out") + GRAD_NAMES, (hT1, out1) + tuple(g1), full):
+            b = b[:, h:h + 1] if name in ("hidden_final", "dhidden_init") else b[:, :, h:h + 1]
+            assert torch.equal(a, b), f"head {h} alone differs from the full run in {name}"
+
+
+def test_chunk_vmap_forward_and_gradient():
+    """Batching as the reference does it (jax.vmap over a leading axis of all five arrays, then the gradient
+    of a scalar loss, gla.py:1331-1344): torch.func.vmap(chunk_gla) equals the batched call bit for bit, in
+    the outputs and in every gradient taken through it; a mapped axis other than 0 and an unmapped
+    hidden_init work too."""
+    from gla_jax_amd import chunk_gla
+    dtype = torch.bfloat16
+    (h0, g, v, k, q), dev = gpu_inputs(3, 128, 2, 64, 3.0, seed=8, dtype=dtype)
+    dhT, dout = cotangents(h0, v, 8, dtype)
+    one = lambda *a: chunk_gla(*a, 64)
+    ref = [t.clone().requires_grad_(True) for t in dev]
+    hT_b, out_b = chunk_gla(*ref, 64)
+    g_b = torch.autograd.grad(loss_of(hT_b, out_b, dhT, dout), ref)
+    mapped = [t.clone().requires_grad_(True) for t in dev]
+    hT_v, out_v = torch.func.vmap(one)(*mapped)
+    assert torch.equal(hT_v, hT_b) and torch.equal(out_v, out_b)
+    g_v = torch.autograd.grad(loss_of(hT_v, out_v, dhT, dout), mapped)
+    for a, b in zip(g_v, g_b):
+        assert torch.equal(a, b)
+    # functional form: grad of (loss of vmap), all five arguments
+    wdh, wdo = to_dev(dhT, torch.float32), to_dev(dout, torch.float32)
+
+    def loss(*a):
+        hT, out = torch.func.vmap(one)(*a)
+        return (hT.float() * wdh).sum() + (out.float() * wdo).sum()
+    g_f = torch.func.grad(loss, argnums=(0, 1, 2, 3, 4))(*dev)
+    for a, b in zip(g_f, g_b):
+        assert torch.equal(a, b)
+    # the sequence arrays mapped over axis 1, one hidden_init shared by the whole batch
+    moved = [dev[0][0]] + [t.movedim(0, 1).contiguous() for t in dev[1:]]
+    hT_m, out_m = torch.func.vmap(one, in_dims=(None, 1, 1, 1, 1))(*moved)
+    hT_s, out_s = chunk_gla(dev[0][0].expand(3, -1, -1, -1).contiguous(), *dev[1:], 64)
+    assert torch.equal(hT_m, hT_s) and torch.equal(out_m, out_s)

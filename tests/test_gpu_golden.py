@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from tests.test_golden import GRADS, INPUTS, load
-from tests.util import TOL, assert_close, err_over_rms, grad_kinds, to_dev, to_np
+from tests.util import GRAD_NAMES, TOL, check_chunk_outputs, check_recurrent_outputs, err_over_rms, to_dev, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -15,12 +15,10 @@ def device_inputs(d, dtype):
     return [to_dev(d[k], torch.float32 if k == "log_fgate" else dtype) for k in INPUTS]
 
 
-def check(d, tag, dtype, hT, out, grads):
-    tol = TOL[dtype]
-    assert_close("out", to_np(out), d[f"{tag}_out"], tol, stored=dtype)
-    assert_close("hidden_final", to_np(hT), d[f"{tag}_hidden_final"], tol, stored=dtype)
-    for name, got, st in zip(GRADS, grads, grad_kinds(dtype)):
-        assert_close(name, to_np(got), d[f"{tag}_{name}"], tol, stored=st)
+def golden(d, tag):
+    """(dh0, dg, dv, dk, dq, hidden_final, out) of the fixture, in the oracle's order."""
+    assert tuple(GRADS) == GRAD_NAMES
+    return tuple(d[f"{tag}_{n}"] for n in GRADS) + (d[f"{tag}_hidden_final"], d[f"{tag}_out"])
 
 
 def fwd_bwd(fn, d, dtype, **kw):
@@ -37,7 +35,10 @@ def test_chunk_gla_against_golden(dtype, chunk):
     from gla_jax_amd import chunk_gla
     d = load("gla_T64_H1_D64.npz")
     hT, out, grads = fwd_bwd(chunk_gla, d, dtype, chunk_size=chunk)
-    check(d, "fwd", dtype, hT, out, grads)
+    arrs = tuple(np.asarray(d[k_], dtype=np.float32)[None] for k_ in INPUTS)
+    lead = lambda a: np.asarray(a)[None]
+    check_chunk_outputs(dtype, arrs, chunk, hT[None], out[None], [t[None] for t in grads],
+                        lead(d["dhidden_final"]), lead(d["dout"]), exact=tuple(lead(a) for a in golden(d, "fwd")))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
@@ -46,7 +47,7 @@ def test_recurrent_gla_against_golden(dtype, reverse):
     from gla_jax_amd import recurrent_gla
     d = load("gla_T64_H1_D64.npz")
     hT, out, grads = fwd_bwd(recurrent_gla, d, dtype, reverse=reverse)
-    check(d, "rev" if reverse else "fwd", dtype, hT, out, grads)
+    check_recurrent_outputs(dtype, golden(d, "rev" if reverse else "fwd"), hT, out, grads)
 
 
 @pytest.mark.parametrize("reverse", [False, True])

@@ -7,7 +7,7 @@ import torch
 
 from oracle import gla_oracle as O
 from oracle import naive_c
-from tests.util import TOL, assert_close, cotangents, gpu_inputs, grad_kinds, to_dev, to_np
+from tests.util import (TOL, assert_plain, check_recurrent_outputs, cotangents, fmt_log, gpu_inputs, to_dev, to_np)
 
 pytestmark = pytest.mark.gpu
 
@@ -32,12 +32,7 @@ def test_recurrent_gla_matches_oracle(dtype, B, T, H, D, reverse):
                                  reverse=reverse)
     assert out.dtype == dtype and hT.dtype == dtype
     exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=reverse)
-    tol = TOL[dtype]
-    assert_close("out", to_np(out), exp[6], tol, stored=dtype)
-    assert_close("hidden_final", to_np(hT), exp[5], tol, stored=dtype)
-    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                grad_kinds(dtype)):
-        assert_close(name, to_np(got), e, tol, stored=st)
+    print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads)))
 
 
 @pytest.mark.parametrize("D", [32, 64])
@@ -75,12 +70,7 @@ def test_recurrent_matrix_core_path_over_gate_regimes(T, reverse, D):
     hT, out, grads = run_fwd_bwd(recurrent_gla, dev, to_dev(dhT, dtype), to_dev(dout, dtype), dtype,
                                  reverse=reverse)
     exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=reverse)
-    tol = TOL[dtype]
-    assert_close("out", to_np(out), exp[6], tol, stored=dtype)
-    assert_close("hidden_final", to_np(hT), exp[5], tol, stored=dtype)
-    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                grad_kinds(dtype)):
-        assert_close(name, to_np(got), e, tol, stored=st)
+    print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads)))
 
 
 def test_recurrent_gla_naive_returns_fp32_out():
@@ -93,11 +83,28 @@ def test_recurrent_gla_naive_returns_fp32_out():
                                  torch.float32, reverse=False)
     assert out.dtype == torch.float32 and hT.dtype == dtype            # gla.py:37, 46
     exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout)
-    assert_close("out", to_np(out), exp[6], 1e-4)                      # fp32 state and output
-    assert_close("hidden_final", to_np(hT), exp[5], TOL[dtype], stored=dtype)
-    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                grad_kinds(dtype)):
-        assert_close(name, to_np(got), e, TOL[dtype], stored=st)
+    assert_plain("out", to_np(out), exp[6], 1e-4)                      # fp32 state and output
+    print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads, out_fp32=True)))
+
+
+def test_recurrent_gla_naive_reverse():
+    """recurrent_gla_naive(reverse=True) (gla.py:45): the scan runs from the last step down, outputs stay in
+    place; forward and all gradients."""
+    from gla_jax_amd import recurrent_gla_naive
+    dtype = torch.bfloat16
+    (h0, g, v, k, q), dev = gpu_inputs(2, 77, 3, 64, 2.0, seed=19, dtype=dtype)
+    dhT, dout = cotangents(h0, v, 4, torch.float32)
+    dhT = O.bf16_round(dhT)
+    hT, out, grads = run_fwd_bwd(recurrent_gla_naive, dev, to_dev(dhT, dtype), to_dev(dout, torch.float32),
+                                 torch.float32, reverse=True)
+    assert out.dtype == torch.float32 and hT.dtype == dtype
+    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=True)
+    assert_plain("out", to_np(out), exp[6], 1e-4)
+    print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads, out_fp32=True)))
+    # the reversed scan is the forward scan of the flipped sequence (gla.py:421-438)
+    fl = lambda t: t.flip(1).contiguous()
+    hT2, out2 = recurrent_gla_naive(dev[0], fl(dev[1]), fl(dev[2]), fl(dev[3]), fl(dev[4]), False)
+    assert torch.equal(hT2, hT) and torch.equal(fl(out2), out)
 
 
 def test_recurrent_unbatched_and_vmap_agree():
@@ -121,12 +128,7 @@ def test_recurrent_full_benchmark_shape_against_c_oracle():
     dhT, dout = cotangents(h0, v, 3, dtype)
     hT, out, grads = run_fwd_bwd(recurrent_gla, dev, to_dev(dhT, dtype), to_dev(dout, dtype), dtype)
     exp = naive_c.naive_bwd(h0, g, v, k, q, dhT, dout, dtype=np.float64, nthreads=16)
-    tol = TOL[dtype]
-    assert_close("out", to_np(out), exp[6], tol, stored=dtype)
-    assert_close("hidden_final", to_np(hT), exp[5], tol, stored=dtype)
-    for name, got, e, st in zip(("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), grads, exp[:5],
-                                grad_kinds(dtype)):
-        assert_close(name, to_np(got), e, tol, stored=st)
+    print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads)))
 
 
 def test_recurrent_rejects_bad_arguments():
