@@ -555,7 +555,8 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
     const size_t lds = ((size_t)(3 * C + VR) * LS + (size_t)NB * 16 * XS) * sizeof(T) +
                        (size_t)(3 * NB + 1) * D * sizeof(float);
     auto kern = chunk_grad_kernel<T, C, D>;
-    if (int e = allow_lds((const void *)kern, lds)) return e;
+    static LdsGrant grant;
+    if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(T_len / C * H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
                        (const T *)dout, (const T *)statesN, (const T *)dstatesT, (const T *)dstatesN, dg,

@@ -174,7 +174,8 @@ int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, co
     constexpr int LS = TileGeom<T, D>::kStride;
     const size_t lds = (size_t)(2 * C - 16 + 32) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
     auto kern = chunk_out_kernel<T, C, D>;
-    if (int e = allow_lds((const void *)kern, lds)) return e;
+    static LdsGrant grant;
+    if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(T_len / C * H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
                        (const T *)states, (T *)out, T_len, H);

@@ -247,11 +247,13 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
     dim3 grid(T_len / C * H, B), block(C * 4);
     if (mode == 0) {
         auto kern = chunk_outer_kernel<T, C, D, 0>;
-        if (int e = allow_lds((const void *)kern, lds)) return e;
+        static LdsGrant grant;
+        if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
         hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)x, (const T *)y, prodT, decay, T_len, H);
     } else {
         auto kern = chunk_outer_kernel<T, C, D, 1>;
-        if (int e = allow_lds((const void *)kern, lds)) return e;
+        static LdsGrant grant;
+        if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
         hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)x, (const T *)y, prodT, decay, T_len, H);
     }
     return launch_status();

@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include <type_traits>
 
 #include "../../include/gla_hip.h"
@@ -131,12 +132,25 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
 
-// Dynamic LDS above 64 KB has to be granted per kernel before the launch (gfx950 has 160 KB per CU).
-inline int allow_lds(const void *kernel, size_t bytes)
+// Dynamic LDS above 64 KB has to be granted per kernel before the launch (gfx950 has 160 KB per CU).  The grant
+// sticks to the kernel on the device it was made on, so it is made once per (kernel, device): every launcher
+// keeps one LdsGrant per kernel it launches, a bit per device index.  This and the per-device address of the
+// static scratch array are the only state the library keeps between calls.
+struct LdsGrant {
+    std::atomic<uint64_t> done{0};
+};
+inline int allow_lds(LdsGrant &grant, const void *kernel, size_t bytes)
 {
     if (bytes <= 65536) return 0;
-    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    return e == hipSuccess ? 0 : (int)e;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    const uint64_t bit = dev < 64 ? (1ull << dev) : 0;
+    if (bit && (grant.done.load(std::memory_order_acquire) & bit)) return 0;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return (int)e;
+    grant.done.fetch_or(bit, std::memory_order_release);
+    return 0;
 }
 
 inline int launch_status()

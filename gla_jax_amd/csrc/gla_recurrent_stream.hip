@@ -257,7 +257,8 @@ static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, cons
     constexpr int LS = TileGeom<T, D>::kStride;
     const size_t lds = (size_t)(3 * C + 2 * D) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
     auto kern = recurrent_stream_fwd_kernel<TO, C, D>;
-    if (int e = allow_lds((const void *)kern, lds)) return e;
+    static LdsGrant grant;
+    if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,
                        (T *)hT, (TO *)out, T_len, H, reverse);

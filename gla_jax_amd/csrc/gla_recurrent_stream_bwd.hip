@@ -928,7 +928,8 @@ static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, const
     const size_t lds = ((size_t)(3 * C + 2 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
                        (size_t)(C / 16) * D * sizeof(float);
     auto kern = recurrent_stream_dq_kernel<C, D>;
-    if (int e = allow_lds((const void *)kern, lds)) return e;
+    static LdsGrant grant;
+    if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,
                        (const T *)dhT, (const T *)dout, (T *)dq, qdq, T_len, H, reverse);
@@ -946,7 +947,8 @@ static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, cons
     const size_t lds = ((size_t)(3 * C + 2 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
                        (size_t)(2 * (C / 16) + 2) * D * sizeof(float);
     auto kern = recurrent_stream_rev_kernel<C, D>;
-    if (int e = allow_lds((const void *)kern, lds)) return e;
+    static LdsGrant grant;
+    if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
                        (const T *)dhT, (const T *)dout, (T *)dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse);
