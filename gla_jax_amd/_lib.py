@@ -11,6 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgla_hip.so")
 
 GLA_F32, GLA_BF16 = 0, 1
+GLA_CHUNK_FWD_STATIC_BYTES = 80 << 20      # capacity of gla_chunk_fwd_static's workspace (gla_hip.h)
 
 _i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 
@@ -27,6 +28,7 @@ SIGNATURES = {
     "gla_chunk_bwd_workspace_bytes": (_sz, [_i64] * 6 + [_int]),
     "gla_chunk_fwd": (_int, [_vp] + [_i64] * 6 + [_int] + [_vp] * 9 + [_sz]),
     "gla_chunk_bwd": (_int, [_vp] + [_i64] * 6 + [_int] + [_vp] * 13 + [_sz]),
+    "gla_chunk_fwd_static": (_int, [_vp] + [_i64] * 6 + [_int] + [_vp] * 8),
     "gla_chunk_fwd_stages": (_int, [_vp, _int] + [_i64] * 6 + [_int] + [_vp] * 9 + [_sz]),
     "gla_chunk_bwd_stages": (_int, [_vp, _int] + [_i64] * 6 + [_int] + [_vp] * 13 + [_sz]),
 }

@@ -5,6 +5,8 @@
 //                             ->  grad (dq, dk, dv, dlog_fgate)
 #include "gla_chunk_kernels.hpp"
 
+#include <atomic>
+
 namespace gla {
 
 struct ChunkPlan {
@@ -57,6 +59,34 @@ template <typename F> static int dispatch(int dtype, int C, int D, F &&f)
     GLA_FOR_EACH_CHUNK_CONFIG(GLA_DISPATCH_CASE)
 #undef GLA_DISPATCH_CASE
     return GLA_ERR_UNSUPPORTED;
+}
+
+// ---- the statically allocated workspace of gla_chunk_fwd_static ---------------------------------------------
+// Device memory that belongs to the library's code object: every GPU the library runs on holds its own copy,
+// at its own address, from the moment the code object is loaded there until the process ends.  In host code
+// the array's name is only a handle for hipGetSymbolAddress; the address that kernels and copies may use is
+// looked up once per device (with that device current) and kept in g_scratch_ptr.
+constexpr size_t kStaticScratchBytes = GLA_CHUNK_FWD_STATIC_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+static int static_scratch(void **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return GLA_ERR_UNSUPPORTED;
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return GLA_ERR_WORKSPACE;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);   // two racing first calls store the same address
+    }
+    *out = p;
+    return GLA_OK;
 }
 
 }  // namespace gla
@@ -133,6 +163,24 @@ extern "C" int gla_chunk_fwd(void *stream, int64_t B, int64_t T, int64_t H, int6
 {
     return gla_chunk_fwd_stages(stream, 7, B, T, H, DK, DV, chunk_size, dtype, hidden_init, log_fgate, value,
                                 key, query, hidden_final, out, states, workspace, workspace_bytes);
+}
+
+extern "C" int gla_chunk_fwd_static(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                    int64_t chunk_size, gla_dtype dtype, const void *hidden_init,
+                                    const float *log_fgate, const void *value, const void *key,
+                                    const void *query, void *hidden_final, void *out, void *states)
+{
+    ChunkPlan p;
+    int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p);
+    if (rc) return rc;
+    if (p.prod + p.decay + p.states > kStaticScratchBytes) return GLA_ERR_WORKSPACE;   // beyond the static array
+    void *ws = nullptr;
+    rc = static_scratch(&ws);
+    if (rc) return rc;
+    // the workspace needs no clearing: the per-chunk products and decays are written by the first kernel
+    // before the scan reads them, the chunk-start states by the scan before the output kernel reads them
+    return gla_chunk_fwd_stages(stream, 7, B, T, H, DK, DV, chunk_size, dtype, hidden_init, log_fgate, value, key,
+                                query, hidden_final, out, states, ws, kStaticScratchBytes);
 }
 
 extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK,

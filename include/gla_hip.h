@@ -17,7 +17,9 @@
  *   - The library never allocates, frees or synchronises: outputs and workspaces are the caller's.
  *   - Return value: 0 = enqueued; < 0 = argument rejected on the host before any launch (see
  *     gla_status); > 0 = a hipError_t from a launch.  No C++ exception crosses the boundary.
- *   - Re-entrant; no mutable global state.
+ *   - Re-entrant.  The only state kept between calls is set-up that is done once per device and never
+ *     changes afterwards: the grant of more than 64 KB of LDS to the kernels that need it, and the device
+ *     address of the static scratch array of gla_chunk_fwd_static.
  */
 #ifndef GLA_HIP_H_
 #define GLA_HIP_H_
@@ -137,6 +139,24 @@ int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int
                   const void *states, const void *dhidden_final, const void *dout,
                   void *dhidden_init, float *dlog_fgate, void *dvalue, void *dkey, void *dquery,
                   void *workspace, size_t workspace_bytes);
+
+/* gla_chunk_fwd for callers that cannot allocate device memory and have no workspace to pass: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments and results as gla_chunk_fwd without the workspace pair: the per-chunk products,
+ * decays and chunk-start states go through a static device array of GLA_CHUNK_FWD_STATIC_BYTES bytes
+ * (80 MiB: the headline shape B4 T4096 H6 D128 bf16 needs 72.4 MiB) that every GPU the library runs on holds
+ * from the first call on it until the process ends.  Shapes whose workspace (gla_chunk_fwd_workspace_bytes)
+ * exceeds the capacity are rejected with GLA_ERR_WORKSPACE before anything is launched.  The call allocates
+ * and frees nothing.  The first call on a device looks up the array's address there (hipGetSymbolAddress):
+ * make it outside a graph capture.  All calls on one GPU share the one array: calls that overlap in time on
+ * the same GPU (different streams, different host threads) race and must be serialised by the caller; calls
+ * in order on one stream are safe, nothing in the array has to survive from one call to the next. */
+#define GLA_CHUNK_FWD_STATIC_BYTES ((size_t)80 << 20)
+int gla_chunk_fwd_static(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                         int64_t chunk_size, gla_dtype dtype,
+                         const void *hidden_init, const float *log_fgate, const void *value,
+                         const void *key, const void *query,
+                         void *hidden_final, void *out, void *states);
 
 /* Same as gla_chunk_fwd / gla_chunk_bwd but launching only the kernels selected by `stages`
  * (bit 0: per-chunk outer products, bit 1: scan over chunks, bit 2: output / gradient kernel), the

@@ -1,0 +1,60 @@
+"""gla_chunk_fwd_static, the forward entry point that allocates nothing (its workspace is a static device
+array inside the library), through the C ABI against gla_chunk_fwd with a caller-allocated workspace: bit-equal
+outputs on two calls in a row, the second on a smaller input, then on the largest shape that fits; shapes
+beyond the static array are rejected before any launch."""
+import pytest
+import torch
+
+from tests.util import gpu_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_pair(lib, _lib, B, T, H, D, chunk, seed, dtype=torch.bfloat16):
+    _, dev = gpu_inputs(B, T, H, D, 2.0, seed=seed, dtype=dtype)
+    h0, g, v, k, q = dev
+    dt = _lib.GLA_BF16 if dtype == torch.bfloat16 else _lib.GLA_F32
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda t: t.data_ptr()
+    wsb = lib.gla_chunk_fwd_workspace_bytes(B, T, H, D, D, chunk, dt)
+    stb = lib.gla_chunk_states_bytes(B, T, H, D, D, chunk, dt)
+    assert 0 < wsb <= _lib.GLA_CHUNK_FWD_STATIC_BYTES
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    outs = []
+    for static in (False, True):
+        hT, out = torch.full_like(h0, float("nan")), torch.full_like(v, float("nan"))
+        states = torch.zeros(stb, dtype=torch.uint8, device="cuda")
+        if static:
+            rc = lib.gla_chunk_fwd_static(st, B, T, H, D, D, chunk, dt, p(h0), p(g), p(v), p(k), p(q), p(hT), p(out),
+                                          p(states))
+        else:
+            rc = lib.gla_chunk_fwd(st, B, T, H, D, D, chunk, dt, p(h0), p(g), p(v), p(k), p(q), p(hT), p(out),
+                                   p(states), p(ws), wsb)
+        _lib.check("gla_chunk_fwd_static" if static else "gla_chunk_fwd", rc)
+        outs.append((hT, out, states))
+    torch.cuda.synchronize()
+    for name, a, b in zip(("hidden_final", "out", "states"), outs[0], outs[1]):
+        assert torch.isfinite(a.float()).all() if a.dtype != torch.uint8 else True
+        assert torch.equal(a, b), f"{name} of gla_chunk_fwd_static differs from gla_chunk_fwd at {(B, T, H, D)}"
+
+
+def test_static_entry_point_matches_the_workspace_one():
+    from gla_jax_amd import _lib
+    lib = _lib.load()
+    _run_pair(lib, _lib, 2, 512, 3, 128, 128, seed=21)           # first call on this device: looks the array up
+    _run_pair(lib, _lib, 1, 128, 2, 64, 64, seed=22)             # a smaller input right after: stale contents around it
+    _run_pair(lib, _lib, 2, 96, 1, 64, 32, seed=23, dtype=torch.float32)
+    _run_pair(lib, _lib, 4, 4096, 6, 128, 128, seed=24)          # the headline shape: 72.4 of the 80 MiB
+
+
+def test_static_entry_point_rejects_what_does_not_fit():
+    from gla_jax_amd import _lib
+    lib = _lib.load()
+    B, T, H, D = 8, 4096, 6, 128                                  # needs 144.75 MiB
+    assert lib.gla_chunk_fwd_workspace_bytes(B, T, H, D, D, 128, _lib.GLA_BF16) > _lib.GLA_CHUNK_FWD_STATIC_BYTES
+    x = torch.zeros(16, device="cuda")                             # never touched: the call is refused on the host
+    rc = lib.gla_chunk_fwd_static(torch.cuda.current_stream().cuda_stream, B, T, H, D, D, 128, _lib.GLA_BF16,
+                                  *([x.data_ptr()] * 8))
+    assert rc == -5
+    with pytest.raises(_lib.GlaError, match="workspace"):
+        _lib.check("gla_chunk_fwd_static", rc)
