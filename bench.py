@@ -34,8 +34,29 @@ FP32_VALU_PEAK_TFLOPS = 157.3
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (scaled by what the same counters read for a 256 MiB device copy); the runs and their figures
-# are summarised under profiles/.  Keyed by (kernel, B, T, H, D, chunk); absent = not measured.
-MEASURED_TRAFFIC = {("chunk_grad_kernel", 4, 4096, 6, 128, 128): 428.9e6}
+# are summarised under profiles/.  A figure belongs to the kernel source it was measured on: the key carries
+# the first 12 hex digits of the SHA-256 of the kernel's source files (KERNEL_SOURCES), and a kernel whose
+# sources have changed since reports `traffic: null` instead of a stale number.
+KERNEL_SOURCES = {
+    "chunk_grad_kernel": ("gla_chunk_bwd.hip", "gla_chunk_common.hpp", "gla_common.hpp"),
+}
+MEASURED_TRAFFIC = {
+    # (kernel, B, T, H, D, chunk, source hash): bytes per launch
+    ("chunk_grad_kernel", 4, 4096, 6, 128, 128, "000000000000"): 428.9e6,
+}
+
+
+def source_hash(kernel):
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES.get(kernel, ()):
+        with open(os.path.join(ROOT, "gla_jax_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:12]
+
+
+def measured_traffic(kernel, B, T, H, D, chunk):
+    return MEASURED_TRAFFIC.get((kernel, B, T, H, D, chunk, source_hash(kernel)))
 
 WORKLOADS = {
     # name: (kind, B, T, H, D, chunk, gate shift)
@@ -75,7 +96,7 @@ def time_events(fn, steps, warmup):
     return a.elapsed_time(b) / steps
 
 
-def bench_chunk(B, T, H, D, chunk, shift, steps, warmup):
+def bench_chunk(B, T, H, D, chunk, shift, steps, warmup, public=True):
     import torch
     from gla_jax_amd import _lib
     lib = _lib.load()
@@ -114,6 +135,28 @@ def bench_chunk(B, T, H, D, chunk, shift, steps, warmup):
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / steps
 
+    # the same step through the public entry point (torch.autograd.Function, buffers allocated per call)
+    from gla_jax_amd import chunk_gla
+    leaves = [t.clone().requires_grad_(True) for t in (h0, g, v, k, q)] if public else []
+
+    def public_step():
+        hT_, out_ = chunk_gla(*leaves, chunk)
+        torch.autograd.backward((hT_, out_), (dhT, dout))
+        for t in leaves:
+            t.grad = None
+
+    ms_public = None
+    if public:
+        for _ in range(3):
+            public_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(max(steps // 2, 5)):
+            public_step()
+        torch.cuda.synchronize()
+        ms_public = (time.perf_counter() - t0) * 1e3 / max(steps // 2, 5)
+        del leaves
+
     n_th = B * T * H
     N = T // min(chunk, 128)
     state_f32 = B * H * N * D * D * 4
@@ -143,12 +186,13 @@ def bench_chunk(B, T, H, D, chunk, shift, steps, warmup):
         "ms_per_step": ms_step,
         "roofline": {"bound": "hbm", "kernel": dom.split(".")[1], "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((dom.split(".")[1], B, T, H, D, chunk)),
+                     "traffic": measured_traffic(dom.split(".")[1], B, T, H, D, chunk),
                      "alg_bytes_per_launch": dom_alg},
         "kernels": per,
         "step_hbm_frac": round(34 * D * n_th / ms_step / 1e6 / HBM_PEAK_GBS, 4),
         "mfma_frac": round(flops / ms_step / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
         "sum_kernel_ms": round(sum(x["ms"] for x in per.values()), 5),
+        "public_api_ms_per_step": None if ms_public is None else round(ms_public, 5),
     }
     return res
 
@@ -288,6 +332,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="chunk", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="with --workload chunk: skip the short runs of the long-context and recurrent configs")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 3 plain device copies of 256 MiB (a kernel of known traffic, to scale "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
@@ -331,6 +377,23 @@ def main():
         line["dtype"] = "f32"
     elif not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(B, T, H, D, shift)
+    if args.workload == "chunk" and not args.headline_only:
+        # the other BASELINE configs that fit one GPU, each with its own throughput and roofline fraction
+        # (a few steps each; `--workload long|recurrent` gives the full line of one of them)
+        other = {}
+        for name in ("long", "recurrent"):
+            k2, B2, T2, H2, D2, c2, s2 = WORKLOADS[name]
+            n2 = max(5, min(args.steps, 10))
+            r2 = bench_chunk(B2, T2, H2, D2, c2, s2, n2, 2, public=False) if k2 == "chunk" else \
+                bench_recurrent(B2, T2, H2, D2, s2, n2, 2)
+            other[name] = {"workload": f"{'chunk_gla' if k2 == 'chunk' else 'recurrent_gla'} fwd+bwd B{B2} T{T2} H{H2} "
+                                       f"D{D2} bf16, gates log_sigmoid({s2:g}+N(0,1))",
+                           "steps": n2, "ms_per_step": round(r2["ms_per_step"], 5),
+                           "Mtokens_per_s": round(r2["value"], 3), "roofline": r2["roofline"]}
+            for key in ("step_hbm_frac", "mfma_frac", "valu_frac"):
+                if key in r2:
+                    other[name][key] = r2[key]
+        line["other_configs"] = other
     print(json.dumps(line))
 
 
