@@ -31,8 +31,8 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
     if (DK != DV) return GLA_ERR_SHAPE;                      // gla.py:499
     if (!is_pow2(chunk) || T % chunk != 0) return GLA_ERR_CHUNK;   // gla.py:500, 674
     if (chunk < 32) return GLA_ERR_UNSUPPORTED;
-    // largest tile built: 128 tokens for bf16, for fp32 (tiles twice as wide) 64 at D=64 and 32 at D=128
-    int64_t C = dtype == GLA_BF16 ? 128 : (DK > 64 ? 32 : 64);
+    // largest tile built: 128 tokens for bf16 (32 at D=256), for fp32 (tiles twice as wide) 64 at D=64 and 32 at D=128
+    int64_t C = dtype == GLA_BF16 ? (DK > 128 ? 32 : 128) : (DK > 64 ? 32 : 64);
     while (T % C != 0) C /= 2;                               // chunk >= 32 divides T, so this stops at 32 or above
     bool ok = false;
 #define GLA_PLAN_CASE(T_, C_, D_) \

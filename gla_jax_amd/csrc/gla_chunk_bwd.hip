@@ -122,7 +122,8 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 part += dpp_f32<kDppQuadXor1>(part);
                 part += dpp_f32<kDppQuadXor2>(part);
                 part += dpp_f32<kDppRowHalfMirror>(part);
-                if constexpr (D / 8 == 16) part += dpp_f32<kDppRowMirror>(part);
+                if constexpr (D / 8 >= 16) part += dpp_f32<kDppRowMirror>(part);
+                if constexpr (D / 8 == 32) part += shfl_xor_f32(part, 16);   // a row spans two 16-lane groups
                 if (c8 == 0) lbar[32 * slice + row] = part;
             }
         }

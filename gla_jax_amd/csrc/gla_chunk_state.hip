@@ -283,6 +283,7 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hi
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUTER)
 GLA_INST_SCAN(__bf16, 64)
 GLA_INST_SCAN(__bf16, 128)
+GLA_INST_SCAN(__bf16, 256)
 GLA_INST_SCAN(float, 64)
 GLA_INST_SCAN(float, 128)
 

@@ -410,6 +410,7 @@ static int launch_fwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
     case 2: GLA_FWD_CASE(2, 4); break;
     case 4: GLA_FWD_CASE(4, 4); break;
     case 8: GLA_FWD_CASE(8, 2); break;
+    case 16: GLA_FWD_CASE(16, 1); break;
     default: return GLA_ERR_SHAPE;
     }
 #undef GLA_FWD_CASE
@@ -423,19 +424,17 @@ static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
                       const void *dout, void *dh0, float *dg, void *dv, void *dk, void *dq)
 {
     dim3 grid(H, B), block(DK / 16 * 64);
-    // bf16 data at head dimension 64 runs both sweeps on the matrix cores, at 128 sweep 1 only
-    const bool stream1 = sizeof(T) == 2 && sizeof(TO) == 2 && (DK == 64 || DK == 128);
-    if (stream1) {
+    // bf16 data at head dimensions 64 and 128 runs both sweeps on the matrix cores
+    if (sizeof(T) == 2 && sizeof(TO) == 2 && (DK == 64 || DK == 128)) {
         int e = launch_recurrent_stream_dq(st, B, T_len, H, DK, reverse, h0, g, v, k, q, dhT, dout, dq, dg);
         if (e) return e;
         return launch_recurrent_stream_rev(st, B, T_len, H, DK, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
     }
 #define GLA_BWD_CASE(RV_, U_, TB_)                                                                      \
     do {                                                                                                \
-        if (!stream1)                                                                                   \
-            hipLaunchKernelGGL((recurrent_bwd_dq_kernel<T, TO, RV_, U_>), grid, block, 0, st,           \
-                               (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,              \
-                               (const T *)dhT, (const TO *)dout, (T *)dq, dg, T_len, H, reverse);       \
+        hipLaunchKernelGGL((recurrent_bwd_dq_kernel<T, TO, RV_, U_>), grid, block, 0, st,               \
+                           (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,                  \
+                           (const T *)dhT, (const TO *)dout, (T *)dq, dg, T_len, H, reverse);           \
         hipLaunchKernelGGL((recurrent_bwd_rev_kernel<T, TO, RV_, TB_>), grid, block, 0, st, g,          \
                            (const T *)v, (const T *)k, (const T *)q, (const T *)dhT,                    \
                            (const TO *)dout, (T *)dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse);        \
@@ -445,6 +444,7 @@ static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
     case 2: GLA_BWD_CASE(2, 4, 4); break;
     case 4: GLA_BWD_CASE(4, 4, 4); break;
     case 8: GLA_BWD_CASE(8, 2, 2); break;
+    case 16: GLA_BWD_CASE(16, 1, 1); break;
     default: return GLA_ERR_SHAPE;
     }
 #undef GLA_BWD_CASE
@@ -457,7 +457,7 @@ static int check_recurrent(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t 
     if (B <= 0 || T <= 0 || H <= 0 || DK <= 0 || DV <= 0) return GLA_ERR_SHAPE;
     if (B > 65535 || H > 65535 || T > (1 << 30)) return GLA_ERR_SHAPE;
     // the reference requires DK == DV for this path (gla.py:120, 391)
-    if (DK != DV || !(DK == 16 || DK == 32 || DK == 64 || DK == 128)) return GLA_ERR_SHAPE;
+    if (DK != DV || !(DK == 16 || DK == 32 || DK == 64 || DK == 128 || DK == 256)) return GLA_ERR_SHAPE;
     if (dtype != GLA_F32 && dtype != GLA_BF16) return GLA_ERR_DTYPE;
     if (out_dtype != GLA_F32 && out_dtype != GLA_BF16) return GLA_ERR_DTYPE;
     if (out_dtype == GLA_BF16 && dtype == GLA_F32) return GLA_ERR_DTYPE;

@@ -81,7 +81,7 @@ int gla_rnn_scan_f32(void *stream, const float *log_fgate, const float *kv,
  * state is written except hidden_final.  reverse != 0 scans t = T-1..0 with outputs left in place
  * (gla.py:421-438).  out_dtype is the element type of `out` (value dtype for recurrent_gla,
  * GLA_F32 for the recurrent_gla_naive flavour whose output is fp32 by promotion, gla.py:37).
- * Requires DK == DV (gla.py:120) in {16, 32, 64, 128}. */
+ * Requires DK == DV (gla.py:120) in {16, 32, 64, 128, 256}. */
 int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
                       gla_dtype dtype, gla_dtype out_dtype, int reverse,
                       const void *hidden_init, const float *log_fgate, const void *value,

@@ -30,6 +30,8 @@ CASES = [
     (torch.float32, 1, 256, 2, 128, 128, 4.0),      # fp32 at D=128 runs on the 32-token tile
     (torch.bfloat16, 3, 128, 5, 128, 128, 3.0),     # a single chunk per sequence, odd batch and head counts
     (torch.bfloat16, 1, 64, 1, 64, 64, 3.0),
+    (torch.bfloat16, 2, 160, 2, 256, 32, 4.0),      # head dimension 256 (32-token tiles)
+    (torch.bfloat16, 1, 256, 1, 256, 128, 0.0),     # the same under strong decay
 ]
 
 
@@ -128,6 +130,9 @@ def test_chunk_rejects_what_the_reference_rejects():
         chunk_gla(*dev, 64)                 # 96 % 64 != 0 (einops rearrange, gla.py:674)
     with pytest.raises(_lib.GlaError):
         chunk_gla(*dev, 8)                  # below the smallest tile built here
+    (_, _, _, _, _), dev = gpu_inputs(1, 64, 1, 256, 2.0, seed=3, dtype=torch.float32)
+    with pytest.raises(_lib.GlaError):
+        chunk_gla(*dev, 32)                 # fp32 at head dimension 256: its tiles do not fit a CU's LDS
 
 
 def _full_shape_check(B, T, H, D, chunk, shift, seed, plain=()):
