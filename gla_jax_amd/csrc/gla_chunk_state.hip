@@ -32,9 +32,10 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     extern __shared__ __align__(16) unsigned char smem[];
     T *Xn = reinterpret_cast<T *>(smem);
     T *Yn = Xn + C * LS;
-    float *rtab = reinterpret_cast<float *>(Yn + C * LS);   // [NB][D] e^{tau_m}
+    float *ttab = reinterpret_cast<float *>(Yn + C * LS);   // [NB][D] tau_m: gate total of sub-block m (log2 units)
 
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: scalar loop bounds below
     const int r = lane & 15, c = lane >> 4;
     // heads vary fastest over the grid: workgroups that run together touch the same DRAM pages of the
     // [B, T, H, D] arrays (a token's H rows are contiguous)
@@ -58,17 +59,12 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     // side the sum over the LATER rows, tau - l_j: that one is scanned directly (a suffix scan, then one row
     // down) instead of being formed as a difference, which would cancel against a closed gate (g = -200
     // leaves 3e-5 of absolute error in every later prefix).  The row that ends up with the sub-block total
-    // tau (15 for the prefix, 0 for the suffix) publishes e^{tau}.
+    // tau (15 for the prefix, 0 for the suffix) publishes it.
 #pragma unroll
     for (int i = 0; i < NV; ++i) p[i] = MODE == 0 ? suffix_sum_rows(p[i]) : prefix_sum_rows(p[i]);
     if (r == (MODE == 0 ? 0 : 15)) {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            f32x8 t;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) t.v[e] = fast_exp2(p[8 * ks + e]);
-            st8(rtab + w * D + 32 * ks + 8 * c, t);
-        }
+        for (int ks = 0; ks < KS; ++ks) st8(ttab + w * D + 32 * ks + 8 * c, pack8<float>(p + 8 * ks));
     }
     if (MODE == 0) {
 #pragma unroll
@@ -77,33 +73,40 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) st8(Xn + (16 * w + r) * LS + 32 * ks + 8 * c, xf[ks]);
     __syncthreads();
+    // The gate sum from a row to the chunk's end (keys) or from its start (queries) adds the totals of the
+    // sub-blocks after (before) the wave's own; all sums are <= 0, so ONE exponential per element gives the
+    // factor, and the loop bounds are wave-uniform (no per-lane selects).
+    const int m_lo = MODE == 0 ? w + 1 : 0, m_hi = MODE == 0 ? NB : w;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const int d0 = 32 * ks + 8 * c;
-        float f[8], yv[8];
+        float sum[8], yv[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) f[e] = fast_exp2(p[8 * ks + e]);
-        float all[8];
+        for (int e = 0; e < 8; ++e) sum[e] = p[8 * ks + e];
+        for (int m = m_lo; m < m_hi; ++m) {
+            f32x8 t = ld8(ttab + m * D + d0);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) all[e] = 1.f;
-        for (int m = 0; m < NB; ++m) {
-            f32x8 t = ld8(rtab + m * D + d0);
-            const bool use = MODE == 0 ? (m > w) : (m < w);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                f[e] *= use ? t.v[e] : 1.f;
-                all[e] *= t.v[e];
-            }
+            for (int e = 0; e < 8; ++e) sum[e] += t.v[e];
         }
         unpack8(yf[ks], yv);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) yv[e] *= f[e];
+        for (int e = 0; e < 8; ++e) yv[e] *= fast_exp2(sum[e]);
         st8(Yn + (16 * w + r) * LS + d0, pack8<T>(yv));
-        if (w == 0 && r == 0) {
-            f32x8 t;
+    }
+    if (w == 0 && r == 0) {
+        // chunk decay e^{L_end}: the total over all sub-blocks
 #pragma unroll
-            for (int e = 0; e < 8; ++e) t.v[e] = all[e];
-            st8(decay + (((int64_t)b * H + h) * N + n) * D + d0, t);
+        for (int ks = 0; ks < KS; ++ks) {
+            const int d0 = 32 * ks + 8 * c;
+            f32x8 all = ld8(ttab + d0);
+            for (int m = 1; m < NB; ++m) {
+                f32x8 t = ld8(ttab + m * D + d0);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) all.v[e] += t.v[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) all.v[e] = fast_exp2(all.v[e]);
+            st8(decay + (((int64_t)b * H + h) * N + n) * D + d0, all);
         }
     }
     __syncthreads();
