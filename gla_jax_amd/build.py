@@ -48,5 +48,37 @@ def build(verbose: bool = True) -> str:
     return LIB
 
 
+def jaxlib_include():
+    """Directory holding xla/ffi/api/ffi.h (shipped inside jaxlib), or None."""
+    try:
+        import jaxlib
+    except ImportError:
+        return None
+    inc = os.path.join(os.path.dirname(jaxlib.__file__), "include")
+    return inc if os.path.exists(os.path.join(inc, "xla", "ffi", "api", "ffi.h")) else None
+
+
+def build_xla_ffi(verbose: bool = True):
+    """Compiles the XLA FFI handlers (xla_ffi/gla_xla_ffi.cc) against jaxlib's headers and links them with
+    libgla_hip.so.  Returns the path, or None when jaxlib's headers are not installed (then nothing is built:
+    the torch front-end does not need them)."""
+    inc = jaxlib_include()
+    if inc is None:
+        if verbose:
+            print("xla/ffi/api/ffi.h not found (no jaxlib): the XLA FFI handlers are not built")
+        return None
+    src = os.path.join(HERE, "xla_ffi", "gla_xla_ffi.cc")
+    out = os.path.join(HERE, "xla_ffi", "libgla_xla_ffi.so")
+    cmd = [HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-shared", "-I", inc, "-I",
+           os.path.join(HERE, "..", "include"), src, "-o", out, "-L", HERE, "-lgla_hip", "-Wl,-rpath,$ORIGIN/.."]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("XLA FFI handlers failed to build:\n" + r.stderr)
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 if __name__ == "__main__":
     build()
+    build_xla_ffi()
