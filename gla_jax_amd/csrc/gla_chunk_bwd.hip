@@ -71,6 +71,13 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const TrLane<T> Lx = make_tr_lane<T>(XS);
     const int wrow = 16 * w * LS + L.nat;          // this lane's row of a [token][feature] tile
     T *xw = xs + w * 16 * XS;                      // [16][XS]: one 32-feature slice of the wave's rows
+    // a second slice scratch per wave, [16][XS2] (remainders of the own sub-block's operands, bf16 only): in the
+    // rows of the value tile that the staged state rows leave free when the chunk has more than 96 tokens,
+    // behind the tables otherwise
+    constexpr int XS2 = 32;
+    constexpr bool kSpareRows = (C - 96) * LS >= NB * 16 * XS2;
+    T *xw2 = (kSpareRows ? tV + 96 * LS : reinterpret_cast<T *>(lbar + D)) + w * 16 * XS2;
+    const TrLane<T> Lx2 = make_tr_lane<T>(XS2);
 
     // ---- staging of the state operands -----------------------------------------------------------------
     // A slice needs rows 32*slice .. +31 of S_n [dk][dv], dS' [dk][dv] and dS' [dv][dk]: 3 x 32 rows of
@@ -359,7 +366,12 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             dl8[e] = 0.f;
         }
         if (one_anchor) {
-            // the own sub-block is one more link on either side: dq~ = dA k~, dk~ = dA^T q~ (below the diagonal)
+            // the own sub-block is one more link on either side: dq~ = dA k~, dk~ = dA^T q~ (below the diagonal).
+            // Both operands, q e^{l - tau} and k e^{tau - l}, enter as bf16 head + remainder.  With ONE anchor
+            // per sub-block each row has a single rounding of either operand, shared by all of its 15 partners,
+            // and under strong decay the pairs next to the diagonal carry most of the gate gradient: with plain
+            // bf16 operands d(log_fgate) came out 1.2x (up to 2.7x) less accurate than the reference's dyadic
+            // anchors give it (whose operand next to the anchor is exact); with the remainders it is 0.7x.
             f32x8 tau = ld8(ttab + w * D + fo + 8 * c);
             float fq[8], fk[8], x[8], xr[8], kr[8];
 #pragma unroll
@@ -371,21 +383,60 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 x[e] = a[e] * fq[e];
                 kr[e] = bq[e] * fk[e];
             }
-            D8 X = pack8<T>(x);
-            unpack8(X, xr);
-            unpack8(pack8<T>(kr), kr);
-            st8(xw + Lx.nat, X);
-            asm volatile("" ::: "memory");
+            f32x4 gq[2], hk[2];
+            const f32x4 z4 = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (sizeof(T) == 2) {
+                // head + remainder carry 16 bits of mantissa: the multipliers of the gate gradient below are the
+                // unrounded x and k e^{tau-l} themselves (they differ from what the MFMAs see by 2^-17, far below
+                // the rounding of dA; the + and - copy of a pair term need not agree to the last bit)
+                float t8[8];
+                const D8 Xh = pack8<T>(x);
+                unpack8(Xh, t8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    xr[e] = x[e];
+                    t8[e] = x[e] - t8[e];
+                }
+                const D8 Xl = pack8<T>(t8);
+                unpack8(ld8(tK + wrow + fo), t8);             // k e^{tau-l} as the key tile holds it
+#pragma unroll
+                for (int e = 0; e < 8; ++e) t8[e] = kr[e] - t8[e];    // what the tile's rounding left of it
+                const D8 Kl = pack8<T>(t8);
+                st8(xw + Lx.nat, Xh);
+                st8(xw2 + Lx2.nat, Kl);
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    gq[tt] = mma_t(lds_tr4(xw2 + Lx2.k4 + 4 * tt, XS2), symb[0], z4);
+                    gq[tt] = mma_t(lds_tr4(tK + L.k4 + fo + 4 * tt + 16 * w * LS, LS), symb[0], gq[tt]);
+                }
+                asm volatile("" ::: "memory");   // the same scratch rows now take the remainder of the query side
+                st8(xw2 + Lx2.nat, Xl);
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    hk[tt] = mma_t(lds_tr4(xw2 + Lx2.k4 + 4 * tt, XS2), symb[1], z4);
+                    hk[tt] = mma_t(lds_tr4(xw + Lx.k4 + 4 * tt, XS), symb[1], hk[tt]);
+                }
+            } else {
+                const D8 X = pack8<T>(x);
+                unpack8(X, xr);
+                unpack8(ld8(tK + wrow + fo), kr);
+                st8(xw + Lx.nat, X);
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    gq[tt] = mma_t(lds_tr4(tK + L.k4 + fo + 4 * tt + 16 * w * LS, LS), symb[0], z4);
+                    hk[tt] = mma_t(lds_tr4(xw + Lx.k4 + 4 * tt, XS), symb[1], z4);
+                }
+            }
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
-                f32x4 z4 = {0.f, 0.f, 0.f, 0.f};
-                f32x4 gq = mma_t(lds_tr4(tK + L.k4 + fo + 4 * tt + 16 * w * LS, LS), symb[0], z4);
-                f32x4 hk = mma_t(lds_tr4(xw + Lx.k4 + 4 * tt, XS), symb[1], z4);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    dq8[4 * tt + e] += gq[e] * fq[4 * tt + e];
-                    dk8[4 * tt + e] += hk[e] * fk[4 * tt + e];
-                    dl8[4 * tt + e] += gq[e] * xr[4 * tt + e] - hk[e] * kr[4 * tt + e];
+                    dq8[4 * tt + e] += gq[tt][e] * fq[4 * tt + e];
+                    dk8[4 * tt + e] += hk[tt][e] * fk[4 * tt + e];
+                    dl8[4 * tt + e] += gq[tt][e] * xr[4 * tt + e] - hk[tt][e] * kr[4 * tt + e];
                 }
             }
             asm volatile("" ::: "memory");
@@ -473,8 +524,6 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 for (int tt = 0; tt < 2; ++tt)
                     acc[tt] = mma_d(ld8(sDn + L.own + 4 * tt * LS + 32 * k2), vf[k2], acc[tt]);
             }
-            float kr[8];
-            unpack8(ld8(tK + wrow + fo), kr);              // k e^{tau-l} as the MFMAs saw it
 #pragma unroll
             for (int I = NB - 1; I >= 1; --I) {
                 if (I > w) {
@@ -487,12 +536,13 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                     }
                 }
             }
-            float o[8];
+            float o[8], krt[8];
+            unpack8(ld8(tK + wrow + fo), krt);             // k e^{tau-l} as the MFMAs of the chains saw it
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float hacc = acc[e >> 2][e & 3];
                 o[e] = fast_exp2(s8[e]) * hacc + dk8[e];
-                dl8[e] -= kr[e] * hacc;
+                dl8[e] -= krt[e] * hacc;
             }
             st8_once(dk + rowoff + fo + 8 * c, pack8<T>(o));
         }
@@ -554,7 +604,8 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
     constexpr int NB = C / 16;
     constexpr int VR = C > 96 ? C : 96;
     const size_t lds = ((size_t)(3 * C + VR) * LS + (size_t)NB * 16 * XS) * sizeof(T) +
-                       (size_t)(3 * NB + 1) * D * sizeof(float);
+                       (size_t)(3 * NB + 1) * D * sizeof(float) +
+                       ((C - 96) * LS >= NB * 16 * 32 || sizeof(T) != 2 ? 0 : (size_t)NB * 16 * 32 * sizeof(T));
     auto kern = chunk_grad_kernel<T, C, D>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;

@@ -1,7 +1,14 @@
-"""bf16 chunk_gla cases that a randomized sweep (small shapes, gate shifts -2..5, scattered resets) found
-over an earlier, hand-set tolerance: one gradient tensor each whose worst element sat 0.1-20 % above
-`2e-2 RMS + one bf16 ulp of the element`.  They are kept as named cases and held to the tolerance model of
-tests/util.py (north_star's 2e-2 RMS, or 1.5 x the emulated reference's own error on the same inputs)."""
+"""bf16 chunk_gla cases that randomized sweeps (small shapes, gate shifts -2..5, scattered resets) found out of
+bounds, kept as named cases and held to the tolerance model of tests/util.py (north_star's 2e-2 RMS, or 1.5 x
+the emulated reference's own error on the same inputs).
+
+Two families.  The first nine sat 0.1-20 % above an earlier, hand-set tolerance (`2e-2 RMS + one bf16 ulp of the
+element`) in one gradient tensor each.  The other eleven failed the present model in d(log_fgate) only, all under
+strong decay (gate shift 0 or 1): with ONE anchor per 16-token sub-block and plain bf16 operands the gate
+gradient came out up to 2.2 x less accurate than the reference's dyadic anchors give it; the gradient kernel
+now takes the operands of a sub-block's own products as bf16 head + remainder (gla_chunk_bwd.hip), and a
+repeat of both sweeps (330 cases) finds every tensor within the model, the worst ratio to the emulated
+reference being 1.47 (d(log_fgate), at 2.3e-2 RMS)."""
 import numpy as np
 import pytest
 import torch
@@ -28,6 +35,18 @@ SWEEP_CASES = {
                 "dvalue"),
     "s43_c178": (3, 384, 4, 128, 128, 0.0, 678, 178, None, 0.0, "dhidden_init"),
     "s41_c212": (3, 128, 4, 128, 128, 3.0, 712, 212, None, 0.0, "dquery"),
+    # second family: d(log_fgate) under strong decay
+    "s101_c19": (1, 64, 3, 128, 32, 0.0, 101919, 19, [42, 2, 4], -60.0, "dlog_fgate"),
+    "s101_c51": (2, 128, 4, 128, 32, 1.0, 101951, 51, None, 0.0, "dlog_fgate"),
+    "s101_c94": (2, 128, 1, 128, 128, 1.0, 101994, 94, None, 0.0, "dlog_fgate"),
+    "s101_c115": (1, 96, 2, 128, 32, 1.0, 102015, 115, None, 0.0, "dlog_fgate"),
+    "s101_c123": (1, 64, 1, 64, 32, 1.0, 102023, 123, [2, 20, 22], -25.0, "dlog_fgate"),
+    "s101_c136": (2, 32, 2, 64, 32, 0.0, 102036, 136, None, 0.0, "dlog_fgate"),
+    "s101_c165": (1, 512, 4, 128, 128, 0.0, 102065, 165, None, 0.0, "dlog_fgate"),
+    "s101_c180": (1, 64, 1, 64, 32, 0.0, 102080, 180, None, 0.0, "dlog_fgate"),
+    "s202_c1": (2, 576, 2, 128, 64, 1.0, 202901, 1, None, 0.0, "dlog_fgate"),
+    "s202_c6": (1, 768, 1, 64, 128, 0.0, 202906, 6, None, 0.0, "dlog_fgate"),
+    "s202_c88": (2, 896, 4, 256, 128, 1.0, 202988, 88, None, 0.0, "dlog_fgate"),
 }
 
 
