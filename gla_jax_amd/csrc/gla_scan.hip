@@ -169,9 +169,14 @@ __global__ __launch_bounds__(WAVES * 64) void cumsum_cached_kernel(const float *
     }
 }
 
-// One thread = one (k, 4 consecutive v) strip of the state, walked over T in registers; the loads
-// of step n do not depend on the recurrence, so UNROLL of them are kept in flight.
-template <int UNROLL>
+// One thread = one (k, W consecutive v) strip of the state, walked over T in registers; the loads
+// of step n do not depend on the recurrence, so UNROLL of them are kept in flight.  W = 4 (one
+// 16-byte access per step) when V is a multiple of 4, W = 1 for every other V.
+template <int W> struct Strip;
+template <> struct Strip<4> { typedef f32x4 type; };
+template <> struct Strip<1> { typedef float type; };
+
+template <int UNROLL, int W>
 __global__ __launch_bounds__(256) void rnn_scan_kernel(const float *__restrict__ a,
                                                        const float *__restrict__ kv,
                                                        const float *__restrict__ init_a,
@@ -180,27 +185,28 @@ __global__ __launch_bounds__(256) void rnn_scan_kernel(const float *__restrict__
                                                        float *__restrict__ out_x, int64_t T, int64_t K,
                                                        int64_t V, int reverse)
 {
-    const int64_t v4 = V / 4;
+    typedef typename Strip<W>::type X;
+    const int64_t vw = V / W;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= K * v4) return;
+    if (idx >= K * vw) return;
     const int64_t b = blockIdx.y;
-    const int64_t k = idx / v4, vq = idx % v4;
+    const int64_t k = idx / vw, vq = idx % vw;
     const float *ab = a + b * T * K + k;
-    const f32x4 *xb = reinterpret_cast<const f32x4 *>(kv + b * T * K * V + k * V) + vq;
-    f32x4 *ob = reinterpret_cast<f32x4 *>(out_x + b * T * K * V + k * V) + vq;
+    const X *xb = reinterpret_cast<const X *>(kv + b * T * K * V + k * V) + vq;
+    X *ob = reinterpret_cast<X *>(out_x + b * T * K * V + k * V) + vq;
     float *oab = out_a ? out_a + b * T * K + k : nullptr;
-    f32x4 x = {0.f, 0.f, 0.f, 0.f};
-    if (init_kv) x = reinterpret_cast<const f32x4 *>(init_kv + b * K * V + k * V)[vq];
+    X x = X{};
+    if (init_kv) x = reinterpret_cast<const X *>(init_kv + b * K * V + k * V)[vq];
     float ca = init_a ? init_a[b * K + k] : 0.f;
     int64_t s = 0;
     for (; s + UNROLL <= T; s += UNROLL) {
         float av[UNROLL];
-        f32x4 bv[UNROLL];
+        X bv[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             int64_t t = reverse ? T - 1 - (s + u) : s + u;
             av[u] = ab[t * K];
-            bv[u] = xb[t * K * v4];
+            bv[u] = xb[t * K * vw];
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
@@ -208,16 +214,16 @@ __global__ __launch_bounds__(256) void rnn_scan_kernel(const float *__restrict__
             float f = __expf(av[u]);
             x = f * x + bv[u];
             ca += av[u];
-            ob[t * K * v4] = x;
+            ob[t * K * vw] = x;
             if (oab && vq == 0) oab[t * K] = ca;
         }
     }
     for (; s < T; ++s) {
         int64_t t = reverse ? T - 1 - s : s;
         float av = ab[t * K];
-        x = __expf(av) * x + xb[t * K * v4];
+        x = __expf(av) * x + xb[t * K * vw];
         ca += av;
-        ob[t * K * v4] = x;
+        ob[t * K * vw] = x;
         if (oab && vq == 0) oab[t * K] = ca;
     }
 }
@@ -258,12 +264,14 @@ extern "C" int gla_rnn_scan_f32(void *stream, const float *log_fgate, const floa
                                 int64_t K, int64_t V, int reverse)
 {
     if (!log_fgate || !kv || !out_state) return GLA_ERR_NULL;
-    if (batch <= 0 || T <= 0 || K <= 0 || V <= 0 || V % 4 != 0 || batch > 65535) return GLA_ERR_SHAPE;
-    if (!gla::aligned16(kv) || !gla::aligned16(out_state) || (init_kv && !gla::aligned16(init_kv)))
+    if (batch <= 0 || T <= 0 || K <= 0 || V <= 0 || batch > 65535) return GLA_ERR_SHAPE;
+    const bool wide = V % 4 == 0;
+    if (wide && (!gla::aligned16(kv) || !gla::aligned16(out_state) || (init_kv && !gla::aligned16(init_kv))))
         return GLA_ERR_ALIGN;
-    int64_t n = K * (V / 4);
+    int64_t n = K * (wide ? V / 4 : V);
     dim3 grid((unsigned)((n + 255) / 256), (unsigned)batch);
-    hipLaunchKernelGGL(gla::rnn_scan_kernel<8>, grid, dim3(256), 0, (hipStream_t)stream, log_fgate, kv,
-                       init_log_fgate, init_kv, out_log_lambda, out_state, T, K, V, reverse);
+    auto kern = wide ? gla::rnn_scan_kernel<8, 4> : gla::rnn_scan_kernel<8, 1>;
+    hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, log_fgate, kv, init_log_fgate, init_kv,
+                       out_log_lambda, out_state, T, K, V, reverse);
     return gla::launch_status();
 }

@@ -68,7 +68,9 @@ int gla_cumsum_f32(void *stream, const float *src, const float *init, float *dst
  * problems laid out back to back:
  *   forward: x_n = exp(a_n)[:,None]*x_{n-1} + b_n, x_{-1} = init_kv ; reverse: x_n = exp(a_n)*x_{n+1} + b_n.
  * out_log_lambda [T,K] receives the running sum of a (including init_log_fgate), out_state [T,K,V]
- * the states.  init pointers may be NULL (zeros); out_log_lambda may be NULL.  All float32. */
+ * the states.  init pointers may be NULL (zeros); out_log_lambda may be NULL.  All float32.  Any V >= 1:
+ * a multiple of 4 moves 16 bytes per access (kv, init_kv and out_state then 16-byte aligned), other V
+ * one float. */
 int gla_rnn_scan_f32(void *stream, const float *log_fgate, const float *kv,
                      const float *init_log_fgate, const float *init_kv,
                      float *out_log_lambda, float *out_state,

@@ -72,7 +72,8 @@ def test_entry_points_reject_bad_arguments_without_touching_the_gpu():
     assert lib.gla_recurrent_fwd(None, 1, 8, 1, 48, 48, 1, 1, 0, a, a, a, a, a, a, a) == -2
     assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 32, 1, 1, 0, a, a, a, a, a, a, a) == -2   # DK != DV
     assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 5, 1, 0, a, a, a, a, a, a, a) == -3
-    assert lib.gla_rnn_scan_f32(None, a, a, None, None, None, a, 1, 4, 4, 3, 0) == -2          # V % 4
+    assert lib.gla_rnn_scan_f32(None, a, a, None, None, None, a, 1, 4, 4, 0, 0) == -2
+    assert lib.gla_rnn_scan_f32(None, a, a + 4, None, None, None, a, 1, 4, 4, 8, 0) == -6      # 16-byte rows
     # misaligned
     assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 1, 1, 0, a + 2, a, a, a, a, a, a) == -6
     # chunk: not a power of two / not dividing T / unsupported head dim / missing workspace

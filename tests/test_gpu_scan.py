@@ -26,7 +26,8 @@ def test_cumsum_recursive(shape, axis, reverse, with_init):
     assert err_over_rms(to_np(got), exp) < 1e-5
 
 
-@pytest.mark.parametrize("T,K,V,batch", [(32, 128, 128, None), (256, 16, 64, 3), (5, 8, 4, None)])
+@pytest.mark.parametrize("T,K,V,batch", [(32, 128, 128, None), (256, 16, 64, 3), (5, 8, 4, None),
+                                           (19, 5, 7, 2), (9, 3, 1, None), (33, 4, 6, None)])
 @pytest.mark.parametrize("reverse", [False, True])
 @pytest.mark.parametrize("with_init", [False, True])
 def test_rnn_recursive(T, K, V, batch, reverse, with_init):
