@@ -127,6 +127,14 @@ __device__ __forceinline__ float shfl_xor_f32(float v, int mask)
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Workgroup barrier for data exchanged through LDS only: waits for the wave's LDS operations, not for its
+// global loads and stores (`__syncthreads()` waits for those too, i.e. for prefetches that are not needed yet
+// and for streamed stores nobody in the workgroup reads).
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ---- host side ------------------------------------------------------------------------------
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -17,6 +17,11 @@ int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, i
                                const float *g, const void *v, const void *k, const void *q, const void *dhT,
                                const void *dout, void *dq, float *qdq);
 
+// The same sweep with two waves per sub-block (head dimension 64).
+int launch_recurrent_stream_dq2(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
+                                const float *g, const void *v, const void *k, const void *q, const void *dhT,
+                                const void *dout, void *dq, float *qdq);
+
 // Sweep 2: dk, dv, dh0 and dlog_fgate (`dg` holds sweep 1's q*dq on entry).
 int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, const float *g,
                                 const void *v, const void *k, const void *q, const void *dhT,
