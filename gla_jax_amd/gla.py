@@ -61,12 +61,46 @@ def _prep(hidden_init, log_fgate, value, key, query):
         B *= s
     # the state enters the kernels in the value dtype (the reference's chunk path casts it the same way,
     # gla.py:720) and hidden_final goes back out in hidden_init's own dtype (gla.py:46, 727)
-    h0 = hidden_init.reshape(B, H, DK, DV).to(dt).contiguous()
-    g = log_fgate.reshape(B, T, H, DK).to(torch.float32).contiguous()      # gates are fp32 (gla.py:495)
-    v = value.reshape(B, T, H, DV).contiguous()
-    k = key.reshape(B, T, H, DK).contiguous()
-    q = query.reshape(B, T, H, DK).contiguous()
+    h0 = _as(hidden_init, (B, H, DK, DV), dt)
+    g = _as(log_fgate, (B, T, H, DK), torch.float32)                       # gates are fp32 (gla.py:495)
+    v = _as(value, (B, T, H, DV), dt)
+    k = _as(key, (B, T, H, DK), dt)
+    q = _as(query, (B, T, H, DK), dt)
     return (h0, g, v, k, q), lead, (B, T, H, DK, DV)
+
+
+def _as(t, shape, dtype):
+    """`t` dense, in `shape` and `dtype`: the tensor itself when it already is (no op, no autograd node: a step
+    at the benchmark shape is bound by the host, every node costs microseconds), else a differentiable copy."""
+    if tuple(t.shape) == shape and t.dtype == dtype and t.is_contiguous():
+        return t
+    return t.reshape(shape).to(dtype).contiguous()
+
+
+_transforms_active = getattr(torch._C, "_are_functorch_transforms_active", None)
+
+
+def _twin(cls):
+    """A twin of a setup_context-style Function in the older style (forward takes ctx).  `Function.apply` of the
+    newer style binds the arguments through `inspect.signature` on every call (tens of microseconds), which it
+    needs for function transforms only; `_apply` picks the twin when no transform is active."""
+    class Twin(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, *args):
+            out = cls.forward(*args)
+            cls.setup_context(ctx, args, out)
+            return out
+
+        backward = staticmethod(cls.backward)
+
+    Twin.__name__ = Twin.__qualname__ = cls.__name__ + "Twin"
+    return Twin
+
+
+def _apply(cls, *args):
+    if _transforms_active is None or _transforms_active():
+        return cls.apply(*args)
+    return cls._twin.apply(*args)
 
 
 def _merge_mapped(info, in_dims, tensors):
@@ -136,7 +170,7 @@ class _ChunkGLA(torch.autograd.Function):
         DV = v.shape[-1]
         dhT = torch.zeros(B, H, DK, DV, dtype=v.dtype, device=v.device) if dhT is None else dhT
         dout = torch.zeros_like(v) if dout is None else dout
-        return _ChunkGLABwd.apply(states, g, v, k, q, dhT, dout, ctx.chunk_size) + (None,)
+        return _apply(_ChunkGLABwd, states, g, v, k, q, dhT, dout, ctx.chunk_size) + (None,)
 
     @staticmethod
     def vmap(info, in_dims, *args):
@@ -202,8 +236,8 @@ def chunk_gla(hidden_init, log_fgate, value, key, query, chunk_size, block_size_
         raise AssertionError(f"Chunk length must be power of 2, but got {chunk_size}")  # gla.py:500
     if T % chunk_size:
         raise AssertionError(f"sequence length {T} is not a multiple of chunk_size {chunk_size}")
-    hT, out = _ChunkGLA.apply(h0, g, v, k, q, chunk_size)[:2]
-    return hT.reshape(lead + (H, DK, DV)).to(hidden_init.dtype), out.reshape(lead + (T, H, DV))
+    hT, out = _apply(_ChunkGLA, h0, g, v, k, q, chunk_size)[:2]
+    return _as(hT, lead + (H, DK, DV), hidden_init.dtype), _as(out, lead + (T, H, DV), out.dtype)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -242,7 +276,7 @@ class _RecurrentGLA(torch.autograd.Function):
         o_torch = torch.float32 if ctx.out_fp32 else v.dtype
         dhT = torch.zeros_like(h0) if dhT is None else dhT
         dout = torch.zeros(v.shape, dtype=o_torch, device=v.device) if dout is None else dout
-        return _RecurrentGLABwd.apply(h0, g, v, k, q, hT, dhT, dout, ctx.reverse, ctx.out_fp32) + (None, None)
+        return _apply(_RecurrentGLABwd, h0, g, v, k, q, hT, dhT, dout, ctx.reverse, ctx.out_fp32) + (None, None)
 
     @staticmethod
     def vmap(info, in_dims, *args):
@@ -291,8 +325,8 @@ def _recurrent(hidden_init, log_fgate, value, key, query, reverse, out_fp32):
     (h0, g, v, k, q), lead, (B, T, H, DK, DV) = _prep(hidden_init, log_fgate, value, key, query)
     if DK != DV:
         raise AssertionError("Not supported yet: key and value head dims differ")      # gla.py:120, 391
-    hT, out = _RecurrentGLA.apply(h0, g, v, k, q, bool(reverse), bool(out_fp32))
-    return hT.reshape(lead + (H, DK, DV)).to(hidden_init.dtype), out.reshape(lead + (T, H, DV))
+    hT, out = _apply(_RecurrentGLA, h0, g, v, k, q, bool(reverse), bool(out_fp32))
+    return _as(hT, lead + (H, DK, DV), hidden_init.dtype), _as(out, lead + (T, H, DV), out.dtype)
 
 
 def recurrent_gla(hidden_init, log_fgate, value, key, query, reverse: bool = False,
@@ -312,3 +346,7 @@ def recurrent_gla_naive(hidden, log_fgate, value, key, query, reverse):
     (gla.py:46).  On this build it runs the same per-timestep HIP kernel as `recurrent_gla`, writing
     fp32 outputs."""
     return _recurrent(hidden, log_fgate, value, key, query, reverse, True)
+
+
+for _cls in (_ChunkGLA, _ChunkGLABwd, _RecurrentGLA, _RecurrentGLABwd):
+    _cls._twin = _twin(_cls)
