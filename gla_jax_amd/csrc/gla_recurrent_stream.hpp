@@ -27,4 +27,9 @@ int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, 
                                 const void *v, const void *k, const void *q, const void *dhT,
                                 const void *dout, void *dh0, float *dg, void *dv, void *dk);
 
+// The same sweep with two waves per sub-block (head dimension 64).
+int launch_recurrent_stream_rev2(hipStream_t st, int B, int T_len, int H, int D, int reverse, const float *g,
+                                 const void *v, const void *k, const void *q, const void *dhT, const void *dout,
+                                 void *dh0, float *dg, void *dv, void *dk);
+
 }  // namespace gla

@@ -797,7 +797,7 @@ int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, 
                                 const void *v, const void *k, const void *q, const void *dhT,
                                 const void *dout, void *dh0, float *dg, void *dv, void *dk)
 {
-    if (D == 64) return launch_rev<64, 64>(st, B, T_len, H, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
+    if (D == 64) return launch_recurrent_stream_rev2(st, B, T_len, H, D, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
     if (D == 128) return launch_rev<64, 128>(st, B, T_len, H, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
     return GLA_ERR_UNSUPPORTED;
 }
