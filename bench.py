@@ -42,7 +42,7 @@ KERNEL_SOURCES = {
 }
 MEASURED_TRAFFIC = {
     # (kernel, B, T, H, D, chunk, source hash): bytes per launch
-    ("chunk_grad_kernel", 4, 4096, 6, 128, 128, "21896e3c7670"): 427.5e6,
+    ("chunk_grad_kernel", 4, 4096, 6, 128, 128, "bbe7718f33c9"): 427.4e6,
 }
 
 
@@ -237,7 +237,8 @@ def bench_recurrent(B, T, H, D, shift, steps, warmup):
     # (the backward really moves 38*D bytes per token-head: both sweeps read g, q, k, v, dout and q*dq
     # makes an fp32 round trip, as in the reference's two-sweep kernel)
     per = {"recurrent_stream_fwd_kernel": {"ms": round(ms_f, 5), "alg_GBs": round(12 * D * n_th / ms_f / 1e6, 1)},
-           "recurrent_stream_dq_kernel + recurrent_stream_rev_kernel": {
+           ("recurrent_stream_dq2_kernel + recurrent_stream_rev2_kernel" if D == 64 else
+            "recurrent_stream_dq_kernel + recurrent_stream_rev_kernel"): {
                "ms": round(ms_b, 5), "alg_GBs": round(22 * D * n_th / ms_b / 1e6, 1),
                "moved_GBs": round(38 * D * n_th / ms_b / 1e6, 1)}}
     achieved = alg / ms_step / 1e6
