@@ -61,6 +61,8 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
     T *xh = xs + (2 * W) * 16 * XS, *xl = xh + 16 * XS;
     const int N = (T_len + C - 1) / C;
     const int tv = W % NB, nt0 = 2 * (W / NB);     // the wave's state tiles: value tile tv, key tiles nt0, nt0 + 1
+    // the wave with the longer chain of the two on a SIMD goes first when both are ready
+    if (I >= NB / 2) __builtin_amdgcn_s_setprio(1);
 
     // state: S[j][e] = state[dk = 16(nt0 + j) + r][dv = 16 tv + 4c + e]
     f32x4 S[2];
@@ -451,6 +453,8 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
     T *xh = xs + (2 * W) * 16 * XS, *xl = xh + 16 * XS;
     const int N = (T_len + C - 1) / C;
     const int td = W % NB, nt0 = 2 * (W / NB);     // the wave's state tiles: key tile td, value tiles nt0, nt0 + 1
+    // the wave with the longer chains of the two on a SIMD goes first when both are ready
+    if (J0 < NB / 2) __builtin_amdgcn_s_setprio(1);
 
     // dS: DS[j][e] = dS[dk = 16 td + 4c + e][dv = 16(nt0 + j) + r]
     f32x4 DS[2];
