@@ -130,30 +130,36 @@ def _no_double_backward(name):
 # ------------------------------------------------------------------------------------------------
 # chunk_gla
 # ------------------------------------------------------------------------------------------------
+def _chunk_forward(h0, g, v, k, q, chunk_size, residual):
+    """One call of gla_chunk_fwd on canonical arrays; `residual` False: no chunk states are kept."""
+    # the kernels take dense arrays by address; a transform may hand over views (a broadcast hidden_init)
+    h0, g, v, k, q = (t.contiguous() for t in (h0, g, v, k, q))
+    B, T, H, DK = k.shape
+    DV = v.shape[-1]
+    lib = _lib.load()
+    dt = _DT[v.dtype]
+    ws_bytes = lib.gla_chunk_fwd_workspace_bytes(B, T, H, DK, DV, chunk_size, dt)
+    st_bytes = lib.gla_chunk_states_bytes(B, T, H, DK, DV, chunk_size, dt)
+    if ws_bytes == 0 or st_bytes == 0:
+        _lib.check("gla_chunk_fwd", -7)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=v.device)
+    # without a residual (nothing to differentiate) the scan skips the [dk][dv] copy of the chunk states
+    states = torch.empty(st_bytes, dtype=torch.uint8, device=v.device) if residual else None
+    hT = torch.empty_like(h0)
+    out = torch.empty_like(v)
+    rc = lib.gla_chunk_fwd(_stream(), B, T, H, DK, DV, chunk_size, dt, _ptr(h0), _ptr(g), _ptr(v),
+                           _ptr(k), _ptr(q), _ptr(hT), _ptr(out), _ptr(states), _ptr(ws), ws_bytes)
+    _lib.check("gla_chunk_fwd", rc)
+    return hT, out, states
+
+
 class _ChunkGLA(torch.autograd.Function):
     """forward = chunk_gla_forward (gla.py:483-550); backward = chunk_gla_backward (gla.py:552-625).
     Arguments are the canonical arrays of `_prep`."""
 
     @staticmethod
     def forward(h0, g, v, k, q, chunk_size):
-        # the kernels take dense arrays by address; a transform may hand over views (a broadcast hidden_init)
-        h0, g, v, k, q = (t.contiguous() for t in (h0, g, v, k, q))
-        B, T, H, DK = k.shape
-        DV = v.shape[-1]
-        lib = _lib.load()
-        dt = _DT[v.dtype]
-        ws_bytes = lib.gla_chunk_fwd_workspace_bytes(B, T, H, DK, DV, chunk_size, dt)
-        st_bytes = lib.gla_chunk_states_bytes(B, T, H, DK, DV, chunk_size, dt)
-        if ws_bytes == 0 or st_bytes == 0:
-            _lib.check("gla_chunk_fwd", -7)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=v.device)
-        states = torch.empty(st_bytes, dtype=torch.uint8, device=v.device)
-        hT = torch.empty_like(h0)
-        out = torch.empty_like(v)
-        rc = lib.gla_chunk_fwd(_stream(), B, T, H, DK, DV, chunk_size, dt, _ptr(h0), _ptr(g), _ptr(v),
-                               _ptr(k), _ptr(q), _ptr(hT), _ptr(out), _ptr(states), _ptr(ws), ws_bytes)
-        _lib.check("gla_chunk_fwd", rc)
-        return hT, out, states
+        return _chunk_forward(h0, g, v, k, q, chunk_size, True)
 
     @staticmethod
     def setup_context(ctx, inputs, output):
@@ -236,7 +242,11 @@ def chunk_gla(hidden_init, log_fgate, value, key, query, chunk_size, block_size_
         raise AssertionError(f"Chunk length must be power of 2, but got {chunk_size}")  # gla.py:500
     if T % chunk_size:
         raise AssertionError(f"sequence length {T} is not a multiple of chunk_size {chunk_size}")
-    hT, out = _apply(_ChunkGLA, h0, g, v, k, q, chunk_size)[:2]
+    if _transforms_active is not None and not _transforms_active() and not (
+            torch.is_grad_enabled() and any(t.requires_grad for t in (h0, g, v, k, q))):
+        hT, out, _ = _chunk_forward(h0, g, v, k, q, chunk_size, False)
+    else:
+        hT, out = _apply(_ChunkGLA, h0, g, v, k, q, chunk_size)[:2]
     return _as(hT, lead + (H, DK, DV), hidden_init.dtype), _as(out, lead + (T, H, DV), out.dtype)
 
 

@@ -63,3 +63,17 @@ def test_second_order_gradients_raise(name):
     assert all(t.requires_grad for t in first)
     with pytest.raises(NotImplementedError, match="second-order"):
         torch.autograd.grad(sum(t.sum() for t in first), args)
+
+
+def test_chunk_forward_without_gradients_keeps_no_residual():
+    """Under no_grad (or with no argument that requires a gradient) chunk_gla skips the chunk-state residual; the
+    results are those of the differentiable call, bit for bit."""
+    from gla_jax_amd import chunk_gla
+    (h0, g, v, k, q), dev = gpu_inputs(2, 256, 2, 128, 3.0, seed=15, dtype=torch.bfloat16)
+    hT_a, out_a = chunk_gla(*[t.clone().requires_grad_(True) for t in dev], 128)
+    with torch.no_grad():
+        hT_b, out_b = chunk_gla(*dev, 128)
+    hT_c, out_c = chunk_gla(*dev, 128)
+    assert not hT_b.requires_grad and not out_c.requires_grad
+    assert torch.equal(hT_a, hT_b) and torch.equal(out_a, out_b)
+    assert torch.equal(hT_a, hT_c) and torch.equal(out_a, out_c)
