@@ -8,7 +8,13 @@ strong decay (gate shift 0 or 1): with ONE anchor per 16-token sub-block and pla
 gradient came out up to 2.2 x less accurate than the reference's dyadic anchors give it; the gradient kernel
 now takes the operands of a sub-block's own products as bf16 head + remainder (gla_chunk_bwd.hip), and a
 repeat of both sweeps (330 cases) finds every tensor within the model, the worst ratio to the emulated
-reference being 1.47 (d(log_fgate), at 2.3e-2 RMS)."""
+reference being 1.47 (d(log_fgate), at 2.3e-2 RMS).
+
+A third list holds what later sweeps found and what is NOT fixed: one case of some 1 150 (mild gates, three
+chunks) whose d(log_fgate) is 1.56 x the emulated reference's error, 4 % over the model.  Its error is the
+chunk-level term sum_v dS' * S_{n+1} (gla.py:782), formed from chunk states stored in bf16 as the reference
+stores them (gla.py:719, 766); both implementations carry that rounding and the ratio of the two maxima
+scatters around 1.  The case is run and reported, and expected to fail."""
 import numpy as np
 import pytest
 import torch
@@ -50,10 +56,19 @@ SWEEP_CASES = {
 }
 
 
-@pytest.mark.parametrize("case", sorted(SWEEP_CASES))
+# found by a sweep, out of bounds, not fixed (see the module docstring)
+OPEN_CASES = {
+    "s505_c115": (3, 384, 2, 128, 128, 5.0, 506015, 115, None, 0.0, "dlog_fgate"),
+}
+
+
+@pytest.mark.parametrize("case", sorted(SWEEP_CASES) + [
+    pytest.param(c, marks=pytest.mark.xfail(reason="d(log_fgate) 1.56 x the emulated reference (bound 1.5 x): the "
+                                                   "bf16 rounding of the stored chunk states", strict=False))
+    for c in sorted(OPEN_CASES)])
 def test_chunk_sweep_case(case):
     from gla_jax_amd import chunk_gla
-    B, T, H, D, chunk, shift, seed, cseed, rows, val, _ = SWEEP_CASES[case]
+    B, T, H, D, chunk, shift, seed, cseed, rows, val, _ = {**SWEEP_CASES, **OPEN_CASES}[case]
     dtype = torch.bfloat16
     (h0, g, v, k, q), dev = gpu_inputs(B, T, H, D, shift, seed=seed, dtype=dtype)
     if rows is not None:
