@@ -55,7 +55,8 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     float *rtab = reinterpret_cast<float *>(xs + NB * 16 * XS);   // [NB][D] e^{tau_m}
     float *dltab = rtab + NB * D;                  // [NB][D] sub-block sums of the gate-cumsum gradient
     float *ttab = dltab + NB * D;                  // [NB][D] tau_m (log2 units)
-    float *lbar = ttab + NB * D;                   // [D] chunk-level gate gradient
+    float *lbar = ttab + NB * D;                   // [D] chunk-level gate gradient, the part that comes from S_n
+    float *lbtab = lbar + D;                       // [NB][32] ... and per sub-block the part of its rows, one slice
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: scalar branches on it
@@ -76,7 +77,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     // behind the tables otherwise
     constexpr int XS2 = 32;
     constexpr bool kSpareRows = (C - 96) * LS >= NB * 16 * XS2;
-    T *xw2 = (kSpareRows ? tV + 96 * LS : reinterpret_cast<T *>(lbar + D)) + w * 16 * XS2;
+    T *xw2 = (kSpareRows ? tV + 96 * LS : reinterpret_cast<T *>(lbtab + NB * 32)) + w * 16 * XS2;
     const TrLane<T> Lx2 = make_tr_lane<T>(XS2);
 
     // ---- staging of the state operands -----------------------------------------------------------------
@@ -85,7 +86,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     T *sS = tV, *sDn = tV + 32 * LS, *sDt = tV + 64 * LS;
     constexpr int kPieces = 32 * D / 8;                       // 8-element pieces of one staged operand
     constexpr int kPer = (kPieces + C * 4 - 1) / (C * 4);     // pieces per thread
-    D8 pfS[kPer], pfS1[kPer], pfDn[kPer], pfDt[kPer];
+    D8 pfS[kPer], pfDn[kPer], pfDt[kPer];
     f32x8 gN;                                                 // per-row inputs of the next slice
     D8 qN, kN;
     auto stage_fetch = [&](int slice) {
@@ -98,7 +99,6 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             if (kPieces % (C * 4) == 0 || idx < kPieces) {
                 const int off = (32 * slice + idx / (D / 8)) * D + (idx % (D / 8)) * 8;
                 pfS[u] = ld8_once(Sn + off);
-                pfS1[u] = ld8_once(Sn + D * D + off);
                 pfDn[u] = ld8_once(dSn + off);
                 pfDt[u] = ld8_once(dSt + off);
             }
@@ -118,11 +118,12 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 st8(sS + row * LS + c8, pfS[u]);
                 st8(sDn + row * LS + c8, pfDn[u]);
                 st8(sDt + row * LS + c8, pfDt[u]);
-                // chunk-level gate gradient (gla.py:782): both of its terms scale with e^{L_end}, like the state
-                // after the chunk, so it equals sum_v dS' * S_{n+1}.  The D/8 threads that hold one row are
-                // neighbours in a wave.
+                // chunk-level gate gradient (gla.py:782), first term: e^{L_end} sum_v S_n * dS' per key feature.
+                // (The sum of both terms is sum_v dS' * S_{n+1}; formed that way from the stored S_{n+1} it carries
+                // the rounding of a whole state instead of a decayed one, which cost two sweep cases their bound.)
+                // The D/8 threads that hold one row are neighbours in a wave.
                 float x[8], y[8], part = 0.f;
-                unpack8(pfS1[u], x);
+                unpack8(pfS[u], x);
                 unpack8(pfDn[u], y);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) part += x[e] * y[e];
@@ -131,7 +132,12 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 part += dpp_f32<kDppRowHalfMirror>(part);
                 if constexpr (D / 8 >= 16) part += dpp_f32<kDppRowMirror>(part);
                 if constexpr (D / 8 == 32) part += shfl_xor_f32(part, 16);   // a row spans two 16-lane groups
-                if (c8 == 0) lbar[32 * slice + row] = part;
+                if (c8 == 0) {
+                    float lend = 0.f;                            // L_end of the feature, log2 units
+#pragma unroll
+                    for (int m = 0; m < NB; ++m) lend += ttab[m * D + 32 * slice + row];
+                    lbar[32 * slice + row] = part * fast_exp2(lend);
+                }
             }
         }
     };
@@ -524,6 +530,20 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 for (int tt = 0; tt < 2; ++tt)
                     acc[tt] = mma_d(ld8(sDn + L.own + 4 * tt * LS + 32 * k2), vf[k2], acc[tt]);
             }
+            {
+                // second term of the chunk-level gate gradient: sum over the chunk's rows of k e^{L_end - L_j} times
+                // the state term (v_j dS'^T) just formed (the reference's -sum_c dLambda_k, gla.py:776-782); summed
+                // over the wave's 16 rows here, over the sub-blocks after the barrier
+                D8 kts = Kt[0];
+#pragma unroll
+                for (int i = 1; i < KS; ++i) kts = ks == i ? Kt[i] : kts;
+                float kte[8];
+                unpack8(kts, kte);
+                f32x8 tb;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) tb.v[e] = suffix_sum_rows(kte[e] * acc[e >> 2][e & 3]);
+                if (r == 0) st8(lbtab + w * 32 + 8 * c, tb);
+            }
 #pragma unroll
             for (int I = NB - 1; I >= 1; --I) {
                 if (I > w) {
@@ -580,6 +600,20 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             f32x8 o = ld8(lbar + fo + 8 * c);
 #pragma unroll
             for (int e = 0; e < 8; ++e) o.v[e] += sfx.v[e];
+            {
+                // sum of the sub-blocks' shares: the 16 rows of a lane group read one share each (two of them the
+                // same one) and add up inside each half of the group
+                static_assert(NB == 8 || NB == 4 || NB == 2, "one share per lane of a quad, a half row or a pair");
+                f32x8 t = ld8(lbtab + (r & (NB - 1)) * 32 + 8 * c);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float x = t.v[e];
+                    x += dpp_f32<kDppQuadXor1>(x);
+                    if (NB >= 4) x += dpp_f32<kDppQuadXor2>(x);
+                    if (NB >= 8) x += dpp_f32<kDppRowHalfMirror>(x);
+                    o.v[e] += x;
+                }
+            }
             for (int m = w + 1; m < NB; ++m) {
                 f32x8 t = ld8(dltab + m * D + fo + 8 * c);
 #pragma unroll
@@ -604,7 +638,7 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
     constexpr int NB = C / 16;
     constexpr int VR = C > 96 ? C : 96;
     const size_t lds = ((size_t)(3 * C + VR) * LS + (size_t)NB * 16 * XS) * sizeof(T) +
-                       (size_t)(3 * NB + 1) * D * sizeof(float) +
+                       ((size_t)(3 * NB + 1) * D + NB * 32) * sizeof(float) +
                        ((C - 96) * LS >= NB * 16 * 32 || sizeof(T) != 2 ? 0 : (size_t)NB * 16 * 32 * sizeof(T));
     auto kern = chunk_grad_kernel<T, C, D>;
     static LdsGrant grant;
