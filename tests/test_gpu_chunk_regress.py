@@ -14,7 +14,12 @@ A third pair came from later sweeps (some 1 300 cases with other seeds): d(log_f
 emulated reference's error, one with mild and one with strong gates.  Both were the chunk-level term of
 gla.py:782, which the gradient kernel formed as sum_v dS' * S_{n+1} from the STORED state after the chunk: that
 carries the bf16 rounding of a whole state, where the reference's two terms carry the rounding of a decayed
-state and of single key rows.  The kernel now forms the two terms as the reference does (gla_chunk_bwd.hip)."""
+state and of single key rows.  The kernel now forms the two terms as the reference does (gla_chunk_bwd.hip).
+
+What stays open is listed apart and expected to fail: one case of a further 300 whose dvalue sits at 1.505 x the
+emulated reference's error (bound 1.5 x, 0.3 % over).  dvalue's error is the bf16 rounding of the score blocks,
+which the reference rounds the same way (gla.py:1029); the two maxima are independent samples and their ratio
+scatters around 1."""
 import numpy as np
 import pytest
 import torch
@@ -59,10 +64,19 @@ SWEEP_CASES = {
 }
 
 
-@pytest.mark.parametrize("case", sorted(SWEEP_CASES))
+# found by a sweep, out of bounds, not fixed (see the module docstring)
+OPEN_CASES = {
+    "s707_c228": (2, 256, 1, 64, 128, 1.0, 708128, 228, None, 0.0, "dvalue"),
+}
+
+
+@pytest.mark.parametrize("case", sorted(SWEEP_CASES) + [
+    pytest.param(c, marks=pytest.mark.xfail(reason="dvalue 1.505 x the emulated reference (bound 1.5 x): the bf16 "
+                                                   "rounding of the score blocks, shared with the reference",
+                                            strict=False)) for c in sorted(OPEN_CASES)])
 def test_chunk_sweep_case(case):
     from gla_jax_amd import chunk_gla
-    B, T, H, D, chunk, shift, seed, cseed, rows, val, _ = SWEEP_CASES[case]
+    B, T, H, D, chunk, shift, seed, cseed, rows, val, _ = {**SWEEP_CASES, **OPEN_CASES}[case]
     dtype = torch.bfloat16
     (h0, g, v, k, q), dev = gpu_inputs(B, T, H, D, shift, seed=seed, dtype=dtype)
     if rows is not None:
