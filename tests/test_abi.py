@@ -104,3 +104,21 @@ def test_oracle_is_not_imported_by_the_product():
     for f in glob.glob(os.path.join(ROOT, "gla_jax_amd", "*.py")):
         src = open(f).read()
         assert "oracle" not in src, f"{f} mentions the oracle: the product path must not depend on it"
+
+
+def test_canonical_arrays_pass_through_untouched():
+    """The host layer adds no op (and no autograd node) for an array that is already dense, shaped and typed as the
+    kernels take it, and converts everything else differentiably."""
+    import torch
+    from gla_jax_amd import gla
+    t = torch.randn(2, 5, 3, 4, requires_grad=True)
+    assert gla._as(t, (2, 5, 3, 4), torch.float32) is t
+    u = gla._as(t, (10, 3, 4), torch.float32)                    # other shape: a view with a node
+    assert u.shape == (10, 3, 4) and u.grad_fn is not None
+    w = gla._as(t.transpose(0, 1), (5, 2, 3, 4), torch.float32)  # not dense: a copy
+    assert w.is_contiguous() and w.grad_fn is not None
+    b = gla._as(t, (2, 5, 3, 4), torch.bfloat16)
+    assert b.dtype == torch.bfloat16 and b.grad_fn is not None
+    # every Function has a twin in the older style that shares its forward, context and backward
+    for cls in (gla._ChunkGLA, gla._ChunkGLABwd, gla._RecurrentGLA, gla._RecurrentGLABwd):
+        assert issubclass(cls._twin, torch.autograd.Function) and cls._twin.backward is cls.backward
