@@ -112,12 +112,12 @@ def bench_chunk(B, T, H, D, chunk, shift, steps, warmup, public=True):
     p = lambda t: t.data_ptr()
 
     def fwd(stages=7):
-        rc = lib.gla_chunk_fwd_stages(st, stages, B, T, H, D, D, chunk, dt, p(h0), p(g), p(v), p(k), p(q),
+        rc = lib.gla_chunk_fwd_stages(st, stages, B, T, H, D, D, chunk, dt, dt, p(h0), p(g), p(v), p(k), p(q),
                                       p(hT), p(out), p(states), p(wsf), wsf.numel())
         _lib.check("gla_chunk_fwd", rc)
 
     def bwd(stages=7):
-        rc = lib.gla_chunk_bwd_stages(st, stages, B, T, H, D, D, chunk, dt, p(g), p(v), p(k), p(q), p(states),
+        rc = lib.gla_chunk_bwd_stages(st, stages, B, T, H, D, D, chunk, dt, dt, p(g), p(v), p(k), p(q), p(states),
                                       p(dhT), p(dout), p(dh0), p(dg), p(dv), p(dk), p(dq), p(wsb), wsb.numel())
         _lib.check("gla_chunk_bwd", rc)
 
@@ -210,11 +210,11 @@ def bench_recurrent(B, T, H, D, shift, steps, warmup):
     p = lambda t: t.data_ptr()
 
     def fwd():
-        _lib.check("gla_recurrent_fwd", lib.gla_recurrent_fwd(st, B, T, H, D, D, dt, dt, 0, p(h0), p(g), p(v),
+        _lib.check("gla_recurrent_fwd", lib.gla_recurrent_fwd(st, B, T, H, D, D, dt, dt, dt, 0, p(h0), p(g), p(v),
                                                             p(k), p(q), p(hT), p(out)))
 
     def bwd():
-        _lib.check("gla_recurrent_bwd", lib.gla_recurrent_bwd(st, B, T, H, D, D, dt, dt, 0, p(h0), p(g), p(v),
+        _lib.check("gla_recurrent_bwd", lib.gla_recurrent_bwd(st, B, T, H, D, D, dt, dt, dt, 0, p(h0), p(g), p(v),
                                                             p(k), p(q), p(hT), p(dhT), p(dout), p(dh0), p(dg),
                                                             p(dv), p(dk), p(dq)))
 

@@ -11,6 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgla_hip.so")
 
 GLA_F32, GLA_BF16 = 0, 1
+ABI_VERSION = 2                             # GLA_HIP_ABI_VERSION of include/gla_hip.h
 GLA_CHUNK_FWD_STATIC_BYTES = 80 << 20      # capacity of gla_chunk_fwd_static's workspace (gla_hip.h)
 
 _i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
@@ -21,16 +22,16 @@ SIGNATURES = {
     "gla_status_string": (ctypes.c_char_p, [_int]),
     "gla_cumsum_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int]),
     "gla_rnn_scan_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int]),
-    "gla_recurrent_fwd": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int] + [_vp] * 7),
-    "gla_recurrent_bwd": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int] + [_vp] * 13),
+    "gla_recurrent_fwd": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _int] + [_vp] * 7),
+    "gla_recurrent_bwd": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _int] + [_vp] * 13),
     "gla_chunk_states_bytes": (_sz, [_i64] * 6 + [_int]),
     "gla_chunk_fwd_workspace_bytes": (_sz, [_i64] * 6 + [_int]),
     "gla_chunk_bwd_workspace_bytes": (_sz, [_i64] * 6 + [_int]),
-    "gla_chunk_fwd": (_int, [_vp] + [_i64] * 6 + [_int] + [_vp] * 9 + [_sz]),
-    "gla_chunk_bwd": (_int, [_vp] + [_i64] * 6 + [_int] + [_vp] * 13 + [_sz]),
-    "gla_chunk_fwd_static": (_int, [_vp] + [_i64] * 6 + [_int] + [_vp] * 8),
-    "gla_chunk_fwd_stages": (_int, [_vp, _int] + [_i64] * 6 + [_int] + [_vp] * 9 + [_sz]),
-    "gla_chunk_bwd_stages": (_int, [_vp, _int] + [_i64] * 6 + [_int] + [_vp] * 13 + [_sz]),
+    "gla_chunk_fwd": (_int, [_vp] + [_i64] * 6 + [_int, _int] + [_vp] * 9 + [_sz]),
+    "gla_chunk_bwd": (_int, [_vp] + [_i64] * 6 + [_int, _int] + [_vp] * 13 + [_sz]),
+    "gla_chunk_fwd_static": (_int, [_vp] + [_i64] * 6 + [_int, _int] + [_vp] * 8),
+    "gla_chunk_fwd_stages": (_int, [_vp, _int] + [_i64] * 6 + [_int, _int] + [_vp] * 9 + [_sz]),
+    "gla_chunk_bwd_stages": (_int, [_vp, _int] + [_i64] * 6 + [_int, _int] + [_vp] * 13 + [_sz]),
 }
 
 _lib = None
@@ -56,8 +57,9 @@ def load():
         fn = getattr(lib, name)      # AttributeError if the symbol is not exported
         fn.restype = res
         fn.argtypes = args
-    if lib.gla_abi_version() != 1:
-        raise ImportError(f"libgla_hip.so ABI {lib.gla_abi_version()} != 1")
+    if lib.gla_abi_version() != ABI_VERSION:
+        raise ImportError(f"libgla_hip.so ABI {lib.gla_abi_version()} != {ABI_VERSION}: rebuild it "
+                          "(`python -m gla_jax_amd.build`)")
     _lib = lib
     return lib
 

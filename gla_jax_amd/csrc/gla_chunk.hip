@@ -23,8 +23,9 @@ static size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
 // the 128-token one: twice or four times the chunk states).  Sizes below 32 tokens are refused: the leaf
 // of the reference needs 32 rows as well (gla.py:975-977).
 static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, int64_t chunk, int dtype,
-                      ChunkPlan *plan)
+                      ChunkPlan *plan, int hidden_dtype = GLA_BF16)
 {
+    if (hidden_dtype != GLA_F32 && hidden_dtype != GLA_BF16) return GLA_ERR_DTYPE;
     if (B <= 0 || T <= 0 || H <= 0 || DK <= 0 || DV <= 0) return GLA_ERR_SHAPE;
     if (B > 65535 || H > 65535 || T > (1 << 30) || B * H > 0x7fffffffLL) return GLA_ERR_SHAPE;   // grid limits
     if (dtype != GLA_F32 && dtype != GLA_BF16) return GLA_ERR_DTYPE;
@@ -117,13 +118,14 @@ extern "C" size_t gla_chunk_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H,
 }
 
 extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK,
-                                    int64_t DV, int64_t chunk_size, gla_dtype dtype, const void *hidden_init,
+                                    int64_t DV, int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
+                                    const void *hidden_init,
                                     const float *log_fgate, const void *value, const void *key,
                                     const void *query, void *hidden_final, void *out, void *states,
                                     void *workspace, size_t workspace_bytes)
 {
     ChunkPlan p;
-    int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p);
+    int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p, hidden_dtype);
     if (rc) return rc;
     const void *req[] = {hidden_init, log_fgate, value, key, query, hidden_final, out};
     for (const void *ptr : req) {
@@ -146,8 +148,8 @@ extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t
             e = launch_chunk_outer<E, C_, D_>(st, 0, (int)B, (int)T, (int)H, log_fgate, value, key, prodT, decay);
         if (e) return e;
         if (stages & 2)
-            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 0, hidden_init, prodT, decay, statesT, states,
-                                         hidden_final, 1);
+            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 0, hidden_dtype, hidden_init, prodT, decay, statesT,
+                                         states, hidden_final, 1);
         if (e) return e;
         if (stages & 4)
             e = launch_chunk_out<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, statesT, out);
@@ -156,22 +158,23 @@ extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t
 }
 
 extern "C" int gla_chunk_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                             int64_t chunk_size, gla_dtype dtype, const void *hidden_init,
+                             int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype, const void *hidden_init,
                              const float *log_fgate, const void *value, const void *key, const void *query,
                              void *hidden_final, void *out, void *states, void *workspace,
                              size_t workspace_bytes)
 {
-    return gla_chunk_fwd_stages(stream, 7, B, T, H, DK, DV, chunk_size, dtype, hidden_init, log_fgate, value,
-                                key, query, hidden_final, out, states, workspace, workspace_bytes);
+    return gla_chunk_fwd_stages(stream, 7, B, T, H, DK, DV, chunk_size, dtype, hidden_dtype, hidden_init, log_fgate,
+                                value, key, query, hidden_final, out, states, workspace, workspace_bytes);
 }
 
 extern "C" int gla_chunk_fwd_static(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                                    int64_t chunk_size, gla_dtype dtype, const void *hidden_init,
+                                    int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
+                                    const void *hidden_init,
                                     const float *log_fgate, const void *value, const void *key,
                                     const void *query, void *hidden_final, void *out, void *states)
 {
     ChunkPlan p;
-    int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p);
+    int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p, hidden_dtype);
     if (rc) return rc;
     if (p.prod + p.decay + p.states > kStaticScratchBytes) return GLA_ERR_WORKSPACE;   // beyond the static array
     void *ws = nullptr;
@@ -179,19 +182,20 @@ extern "C" int gla_chunk_fwd_static(void *stream, int64_t B, int64_t T, int64_t 
     if (rc) return rc;
     // the workspace needs no clearing: the per-chunk products and decays are written by the first kernel
     // before the scan reads them, the chunk-start states by the scan before the output kernel reads them
-    return gla_chunk_fwd_stages(stream, 7, B, T, H, DK, DV, chunk_size, dtype, hidden_init, log_fgate, value, key,
-                                query, hidden_final, out, states, ws, kStaticScratchBytes);
+    return gla_chunk_fwd_stages(stream, 7, B, T, H, DK, DV, chunk_size, dtype, hidden_dtype, hidden_init, log_fgate,
+                                value, key, query, hidden_final, out, states, ws, kStaticScratchBytes);
 }
 
 extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK,
-                                    int64_t DV, int64_t chunk_size, gla_dtype dtype, const float *log_fgate,
+                                    int64_t DV, int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
+                                    const float *log_fgate,
                                     const void *value, const void *key, const void *query, const void *states,
                                     const void *dhidden_final, const void *dout, void *dhidden_init,
                                     float *dlog_fgate, void *dvalue, void *dkey, void *dquery,
                                     void *workspace, size_t workspace_bytes)
 {
     ChunkPlan p;
-    int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p);
+    int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p, hidden_dtype);
     if (rc) return rc;
     const void *req[] = {log_fgate, value, key, query, states, dhidden_final, dout,
                          dhidden_init, dlog_fgate, dvalue, dkey, dquery};
@@ -216,8 +220,8 @@ extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t
             e = launch_chunk_outer<E, C_, D_>(st, 1, (int)B, (int)T, (int)H, log_fgate, dout, query, prodT, decay);
         if (e) return e;
         if (stages & 2)
-            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 1, dhidden_final, prodT, decay, dstatesT, dstatesN,
-                                         dhidden_init, 0);
+            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 1, hidden_dtype, dhidden_final, prodT, decay, dstatesT,
+                                         dstatesN, dhidden_init, 0);
         if (e) return e;
         if (stages & 4)
             e = launch_chunk_grad<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,
@@ -227,13 +231,14 @@ extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t
 }
 
 extern "C" int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                             int64_t chunk_size, gla_dtype dtype, const float *log_fgate, const void *value,
+                             int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype, const float *log_fgate,
+                             const void *value,
                              const void *key, const void *query, const void *states,
                              const void *dhidden_final, const void *dout, void *dhidden_init,
                              float *dlog_fgate, void *dvalue, void *dkey, void *dquery, void *workspace,
                              size_t workspace_bytes)
 {
-    return gla_chunk_bwd_stages(stream, 7, B, T, H, DK, DV, chunk_size, dtype, log_fgate, value, key, query,
-                                states, dhidden_final, dout, dhidden_init, dlog_fgate, dvalue, dkey, dquery,
+    return gla_chunk_bwd_stages(stream, 7, B, T, H, DK, DV, chunk_size, dtype, hidden_dtype, log_fgate, value, key,
+                                query, states, dhidden_final, dout, dhidden_init, dlog_fgate, dvalue, dkey, dquery,
                                 workspace, workspace_bytes);
 }

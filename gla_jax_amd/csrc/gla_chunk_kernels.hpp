@@ -25,7 +25,8 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
                        const void *y, float *prodT, float *decay);
 
 template <typename T, int D>
-int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hin, const float *prodT,
+// hdt = gla_dtype of hin / hout (hidden_init and hidden_final, or their cotangents)
+int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const void *hin, const float *prodT,
                       const float *decay, void *statesT, void *statesN, void *hout, int tail);
 
 template <typename T, int C, int D>

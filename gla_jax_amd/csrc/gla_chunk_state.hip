@@ -146,11 +146,12 @@ template <> struct Pair<float> { typedef f32x2 type; };
 // U = chunks whose inputs are in flight per thread: 4 when the grid fills the machine, 32 when few (b,h)
 // pairs leave it to the single thread to keep the memory system busy (long sequences, small batch).
 template <typename T, int D, int U>
-__global__ __launch_bounds__(64) void chunk_scan_kernel(const T *__restrict__ hin,
+__global__ __launch_bounds__(64) void chunk_scan_kernel(const void *__restrict__ hin,
                                                          const float *__restrict__ prodT,
                                                          const float *__restrict__ decay,
                                                          T *__restrict__ statesT, T *__restrict__ statesN,
-                                                         T *__restrict__ hout, int N, int reverse, int tail)
+                                                         void *__restrict__ hout, int N, int reverse, int tail,
+                                                         int hdt)
 {
     typedef typename Pair<T>::type P2;
     constexpr int TPD = D / 32;
@@ -167,9 +168,13 @@ __global__ __launch_bounds__(64) void chunk_scan_kernel(const T *__restrict__ hi
     float X[2][2];   // X[i][j] = S[dk0 + j][dv0 + i]
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        P2 t = *reinterpret_cast<const P2 *>(hin + (int64_t)bh * D * D + (dk0 + j) * D + dv0);
-        X[0][j] = (float)t[0];
-        X[1][j] = (float)t[1];
+        // the initial state enters the fp32 running state in its own element type (ops.py:396 takes it uncast,
+        // gla.py:711-716); the chunk-start copy of it below is stored in the element type like every other
+        // chunk-start state (gla.py:720)
+        float t[2];
+        load_hidden<2>(hin, hdt, (int64_t)bh * D * D + (dk0 + j) * D + dv0, t);
+        X[0][j] = t[0];
+        X[1][j] = t[1];
     }
     const float *pp = prodT + (int64_t)bh * N * D * D + dv0 * D + dk0;
     const float *dp = decay + (int64_t)bh * N * D + dk0;
@@ -235,9 +240,8 @@ __global__ __launch_bounds__(64) void chunk_scan_kernel(const T *__restrict__ hi
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        P2 t;
-        t[0] = X[0][j]; t[1] = X[1][j];
-        *reinterpret_cast<P2 *>(hout + (int64_t)bh * D * D + (dk0 + j) * D + dv0) = t;
+        const float t[2] = {X[0][j], X[1][j]};
+        store_hidden<2>(hout, hdt, (int64_t)bh * D * D + (dk0 + j) * D + dv0, t);
     }
 }
 
@@ -263,16 +267,16 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
 }
 
 template <typename T, int D>
-int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hin, const float *prodT,
+int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const void *hin, const float *prodT,
                       const float *decay, void *statesT, void *statesN, void *hout, int tail)
 {
     dim3 grid(BH, (D / 16) * (D / 16)), block(64);
     if ((int64_t)grid.y * BH >= 1024) {      // at least a wave per SIMD
-        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 4>), grid, block, 0, st, (const T *)hin, prodT, decay,
-                           (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 4>), grid, block, 0, st, hin, prodT, decay,
+                           (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt);
     } else {
-        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 32>), grid, block, 0, st, (const T *)hin, prodT, decay,
-                           (T *)statesT, (T *)statesN, (T *)hout, N, reverse, tail);
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 32>), grid, block, 0, st, hin, prodT, decay,
+                           (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt);
     }
     return launch_status();
 }
@@ -281,7 +285,7 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, const void *hi
     template int launch_chunk_outer<T, C, D>(hipStream_t, int, int, int, int, const float *, const void *, \
                                              const void *, float *, float *);
 #define GLA_INST_SCAN(T, D)                                                                           \
-    template int launch_chunk_scan<T, D>(hipStream_t, int, int, int, const void *, const float *,     \
+    template int launch_chunk_scan<T, D>(hipStream_t, int, int, int, int, const void *, const float *, \
                                          const float *, void *, void *, void *, int);
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUTER)
 GLA_INST_SCAN(__bf16, 64)

@@ -43,6 +43,12 @@ __device__ __forceinline__ void load_vec(const T *p, float (&dst)[N])
                 f32x4 t = *reinterpret_cast<const f32x4 *>(p + i);
                 dst[i] = t[0]; dst[i + 1] = t[1]; dst[i + 2] = t[2]; dst[i + 3] = t[3];
             }
+        } else if constexpr (N % 2 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 2) {
+                f32x2 t = *reinterpret_cast<const f32x2 *>(p + i);
+                dst[i] = t[0]; dst[i + 1] = t[1];
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < N; ++i) dst[i] = p[i];
@@ -62,6 +68,12 @@ __device__ __forceinline__ void load_vec(const T *p, float (&dst)[N])
 #pragma unroll
                 for (int j = 0; j < 4; ++j) dst[i + j] = (float)t[j];
             }
+        } else if constexpr (N % 2 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 2) {
+                bf16x2 t = *reinterpret_cast<const bf16x2 *>(p + i);
+                dst[i] = (float)t[0]; dst[i + 1] = (float)t[1];
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < N; ++i) dst[i] = (float)p[i];
@@ -78,6 +90,12 @@ __device__ __forceinline__ void store_vec(T *p, const float (&src)[N])
             for (int i = 0; i < N; i += 4) {
                 f32x4 t = {src[i], src[i + 1], src[i + 2], src[i + 3]};
                 *reinterpret_cast<f32x4 *>(p + i) = t;
+            }
+        } else if constexpr (N % 2 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 2) {
+                f32x2 t = {src[i], src[i + 1]};
+                *reinterpret_cast<f32x2 *>(p + i) = t;
             }
         } else {
 #pragma unroll
@@ -100,11 +118,44 @@ __device__ __forceinline__ void store_vec(T *p, const float (&src)[N])
                 for (int j = 0; j < 4; ++j) t[j] = (__bf16)src[i + j];
                 *reinterpret_cast<bf16x4 *>(p + i) = t;
             }
+        } else if constexpr (N % 2 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 2) {
+                bf16x2 t;
+                t[0] = (__bf16)src[i]; t[1] = (__bf16)src[i + 1];
+                *reinterpret_cast<bf16x2 *>(p + i) = t;
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < N; ++i) p[i] = (__bf16)src[i];
         }
     }
+}
+
+// The state arrays (hidden_init, hidden_final and their cotangents) carry an element type of their own, `hdt`
+// (a gla_dtype, uniform over the launch): the reference loads the initial state in its own dtype into an fp32
+// state and stores the final one back in it, whatever the type of value/key/query (gla.py:44-46, 89-97).
+template <int N>
+__device__ __forceinline__ void load_hidden(const void *base, int hdt, int64_t idx, float (&dst)[N])
+{
+    if (hdt == GLA_F32) load_vec<float, N>(static_cast<const float *>(base) + idx, dst);
+    else load_vec<__bf16, N>(static_cast<const __bf16 *>(base) + idx, dst);
+}
+template <int N>
+__device__ __forceinline__ void store_hidden(void *base, int hdt, int64_t idx, const float (&src)[N])
+{
+    if (hdt == GLA_F32) store_vec<float, N>(static_cast<float *>(base) + idx, src);
+    else store_vec<__bf16, N>(static_cast<__bf16 *>(base) + idx, src);
+}
+
+__device__ __forceinline__ float load_hidden1(const void *base, int hdt, int64_t idx)
+{
+    return hdt == GLA_F32 ? static_cast<const float *>(base)[idx] : (float)static_cast<const __bf16 *>(base)[idx];
+}
+__device__ __forceinline__ void store_hidden1(void *base, int hdt, int64_t idx, float x)
+{
+    if (hdt == GLA_F32) static_cast<float *>(base)[idx] = x;
+    else static_cast<__bf16 *>(base)[idx] = (__bf16)x;
 }
 
 // ---- cross-lane ---------------------------------------------------------------------------------

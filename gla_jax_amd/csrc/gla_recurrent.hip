@@ -67,9 +67,9 @@ __device__ __forceinline__ float reduce_over_c(float x)
 // ------------------------------------------------------------------------------------------------
 template <typename T, typename TO, int RK, int U>
 __global__ __launch_bounds__(RK * 64) void recurrent_fwd_kernel(
-    const T *__restrict__ h0, const float *__restrict__ g, const T *__restrict__ v,
-    const T *__restrict__ k, const T *__restrict__ q, T *__restrict__ hT, TO *__restrict__ out,
-    int T_len, int H, int reverse)
+    const void *__restrict__ h0, const float *__restrict__ g, const T *__restrict__ v,
+    const T *__restrict__ k, const T *__restrict__ q, void *__restrict__ hT, TO *__restrict__ out,
+    int T_len, int H, int reverse, int hdt)
 {
     constexpr int DK = RK * 16, DV = DK;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -80,9 +80,9 @@ __global__ __launch_bounds__(RK * 64) void recurrent_fwd_kernel(
 
     float S[RK][4];
     {
-        const T *hp = h0 + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+        const int64_t ho = bh * DK * DV + (int64_t)dk0 * DV + dv0;
 #pragma unroll
-        for (int i = 0; i < RK; ++i) load_vec<T, 4>(hp + (int64_t)i * DV, S[i]);
+        for (int i = 0; i < RK; ++i) load_hidden<4>(h0, hdt, ho + (int64_t)i * DV, S[i]);
     }
     const int64_t strideK = (int64_t)H * DK, strideV = (int64_t)H * DV;
     const float *gp = g + ((int64_t)b * T_len * H + h) * DK + dk0;
@@ -143,9 +143,9 @@ __global__ __launch_bounds__(RK * 64) void recurrent_fwd_kernel(
         compute(cur[0], step);
     }
     {
-        T *hp = hT + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+        const int64_t ho = bh * DK * DV + (int64_t)dk0 * DV + dv0;
 #pragma unroll
-        for (int i = 0; i < RK; ++i) store_vec<T, 4>(hp + (int64_t)i * DV, S[i]);
+        for (int i = 0; i < RK; ++i) store_hidden<4>(hT, hdt, ho + (int64_t)i * DV, S[i]);
     }
 }
 
@@ -157,9 +157,10 @@ __global__ __launch_bounds__(RK * 64) void recurrent_fwd_kernel(
 // ------------------------------------------------------------------------------------------------
 template <typename T, typename TO, int RV, int U>
 __global__ __launch_bounds__(RV * 64) void recurrent_bwd_dq_kernel(
-    const T *__restrict__ h0, const float *__restrict__ g, const T *__restrict__ v,
-    const T *__restrict__ k, const T *__restrict__ q, const T *__restrict__ dhT,
-    const TO *__restrict__ dout, T *__restrict__ dq, float *__restrict__ qdq, int T_len, int H, int reverse)
+    const void *__restrict__ h0, const float *__restrict__ g, const T *__restrict__ v,
+    const T *__restrict__ k, const T *__restrict__ q, const void *__restrict__ dhT,
+    const TO *__restrict__ dout, T *__restrict__ dq, float *__restrict__ qdq, int T_len, int H, int reverse,
+    int hdt)
 {
     constexpr int DV = RV * 16, DK = DV;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -170,9 +171,9 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_dq_kernel(
 
     float S[4][RV];
     {
-        const T *hp = h0 + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+        const int64_t ho = bh * DK * DV + (int64_t)dk0 * DV + dv0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_vec<T, RV>(hp + (int64_t)i * DV, S[i]);
+        for (int i = 0; i < 4; ++i) load_hidden<RV>(h0, hdt, ho + (int64_t)i * DV, S[i]);
     }
     const int64_t strideK = (int64_t)H * DK, strideV = (int64_t)H * DV;
     const int64_t offK = ((int64_t)b * T_len * H + h) * DK + dk0;
@@ -241,12 +242,12 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_dq_kernel(
     // steps s >= t, so the term is added to q*dq of the LAST step and reaches all of them through sweep 2's
     // running sum.  The lane that adds it is the one that stored that q*dq.
     {
-        const T *dp = dhT + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+        const int64_t ho = bh * DK * DV + (int64_t)dk0 * DV + dv0;
         float f4[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float d[RV], acc = 0.f;
-            load_vec<T, RV>(dp + (int64_t)i * DV, d);
+            load_hidden<RV>(dhT, hdt, ho + (int64_t)i * DV, d);
 #pragma unroll
             for (int j = 0; j < RV; ++j) acc += d[j] * S[i][j];
             f4[i] = reduce_over_c(acc);
@@ -273,9 +274,9 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_dq_kernel(
 template <typename T, typename TO, int RV, int TB>
 __global__ __launch_bounds__(RV * 64) void recurrent_bwd_rev_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k,
-    const T *__restrict__ q, const T *__restrict__ dhT,
-    const TO *__restrict__ dout, T *__restrict__ dh0, float *__restrict__ dg, T *__restrict__ dv,
-    T *__restrict__ dk, int T_len, int H, int reverse)
+    const T *__restrict__ q, const void *__restrict__ dhT,
+    const TO *__restrict__ dout, void *__restrict__ dh0, float *__restrict__ dg, T *__restrict__ dv,
+    T *__restrict__ dk, int T_len, int H, int reverse, int hdt)
 {
     constexpr int DV = RV * 16, DK = DV, NW = RV;
     __shared__ float part[TB * NW * 4 * DV];   // [slot][wave][a][dv]: partial dv of 4 state rows each
@@ -287,10 +288,10 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_rev_kernel(
 
     float D[4][RV], run[4];   // run: sum over the later steps of q*dq - k*dk (sweep 1 put sum_v dhT*hT into the last q*dq)
     {
-        const T *dp = dhT + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+        const int64_t ho = bh * DK * DV + (int64_t)dk0 * DV + dv0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            load_vec<T, RV>(dp + (int64_t)i * DV, D[i]);
+            load_hidden<RV>(dhT, hdt, ho + (int64_t)i * DV, D[i]);
             run[i] = 0.f;
         }
     }
@@ -388,23 +389,23 @@ __global__ __launch_bounds__(RV * 64) void recurrent_bwd_rev_kernel(
         for (int u = 0; u < TB; ++u) cur[u] = nxt[u];
     }
     {
-        T *dp = dh0 + bh * DK * DV + (int64_t)dk0 * DV + dv0;
+        const int64_t ho = bh * DK * DV + (int64_t)dk0 * DV + dv0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) store_vec<T, RV>(dp + (int64_t)i * DV, D[i]);
+        for (int i = 0; i < 4; ++i) store_hidden<RV>(dh0, hdt, ho + (int64_t)i * DV, D[i]);
     }
 }
 
 // ------------------------------------------------------------------------------------------------
 template <typename T, typename TO>
-static int launch_fwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, int reverse,
+static int launch_fwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, int reverse, int hdt,
                       const void *h0, const float *g, const void *v, const void *k, const void *q,
                       void *hT, void *out)
 {
     dim3 grid(H, B), block(DV / 16 * 64);
 #define GLA_FWD_CASE(RK_, U_)                                                                        \
-    hipLaunchKernelGGL((recurrent_fwd_kernel<T, TO, RK_, U_>), grid, block, 0, st, (const T *)h0, g, \
-                       (const T *)v, (const T *)k, (const T *)q, (T *)hT, (TO *)out, T_len, H,       \
-                       reverse)
+    hipLaunchKernelGGL((recurrent_fwd_kernel<T, TO, RK_, U_>), grid, block, 0, st, h0, g,            \
+                       (const T *)v, (const T *)k, (const T *)q, hT, (TO *)out, T_len, H,            \
+                       reverse, hdt)
     switch (DK / 16) {
     case 1: GLA_FWD_CASE(1, 4); break;
     case 2: GLA_FWD_CASE(2, 4); break;
@@ -418,7 +419,7 @@ static int launch_fwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
 }
 
 template <typename T, typename TO>
-static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, int reverse,
+static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, int reverse, int hdt,
                       const void *h0, const float *g, const void *v, const void *k, const void *q,
                       const void * /* hidden_final: recomputed in fp32 by sweep 1 */, const void *dhT,
                       const void *dout, void *dh0, float *dg, void *dv, void *dk, void *dq)
@@ -426,18 +427,21 @@ static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
     dim3 grid(H, B), block(DK / 16 * 64);
     // bf16 data at head dimensions 64 and 128 runs both sweeps on the matrix cores
     if (sizeof(T) == 2 && sizeof(TO) == 2 && (DK == 64 || DK == 128)) {
-        int e = launch_recurrent_stream_dq(st, B, T_len, H, DK, reverse, h0, g, v, k, q, dhT, dout, dq, dg);
+        const int dout_f32 = sizeof(TO) == 4;
+        int e = launch_recurrent_stream_dq(st, B, T_len, H, DK, reverse, hdt, dout_f32, h0, g, v, k, q, dhT, dout, dq,
+                                           dg);
         if (e) return e;
-        return launch_recurrent_stream_rev(st, B, T_len, H, DK, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
+        return launch_recurrent_stream_rev(st, B, T_len, H, DK, reverse, hdt, dout_f32, g, v, k, q, dhT, dout, dh0, dg,
+                                           dv, dk);
     }
 #define GLA_BWD_CASE(RV_, U_, TB_)                                                                      \
     do {                                                                                                \
         hipLaunchKernelGGL((recurrent_bwd_dq_kernel<T, TO, RV_, U_>), grid, block, 0, st,               \
-                           (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,                  \
-                           (const T *)dhT, (const TO *)dout, (T *)dq, dg, T_len, H, reverse);           \
+                           h0, g, (const T *)v, (const T *)k, (const T *)q,                             \
+                           dhT, (const TO *)dout, (T *)dq, dg, T_len, H, reverse, hdt);                 \
         hipLaunchKernelGGL((recurrent_bwd_rev_kernel<T, TO, RV_, TB_>), grid, block, 0, st, g,          \
-                           (const T *)v, (const T *)k, (const T *)q, (const T *)dhT,                    \
-                           (const TO *)dout, (T *)dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse);        \
+                           (const T *)v, (const T *)k, (const T *)q, dhT,                               \
+                           (const TO *)dout, dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse, hdt);        \
     } while (0)
     switch (DV / 16) {
     case 1: GLA_BWD_CASE(1, 4, 4); break;
@@ -452,8 +456,9 @@ static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
 }
 
 static int check_recurrent(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, int dtype,
-                           int out_dtype)
+                           int hidden_dtype, int out_dtype)
 {
+    if (hidden_dtype != GLA_F32 && hidden_dtype != GLA_BF16) return GLA_ERR_DTYPE;
     if (B <= 0 || T <= 0 || H <= 0 || DK <= 0 || DV <= 0) return GLA_ERR_SHAPE;
     if (B > 65535 || H > 65535 || T > (1 << 30)) return GLA_ERR_SHAPE;
     // the reference requires DK == DV for this path (gla.py:120, 391)
@@ -467,11 +472,11 @@ static int check_recurrent(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t 
 }  // namespace gla
 
 extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                                 gla_dtype dtype, gla_dtype out_dtype, int reverse,
+                                 gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
                                  const void *hidden_init, const float *log_fgate, const void *value,
                                  const void *key, const void *query, void *hidden_final, void *out)
 {
-    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, out_dtype);
+    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, hidden_dtype, out_dtype);
     if (rc) return rc;
     if (!hidden_init || !log_fgate || !value || !key || !query || !hidden_final || !out)
         return GLA_ERR_NULL;
@@ -479,29 +484,33 @@ extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, 
     for (const void *p : ptrs)
         if (!gla::aligned16(p)) return GLA_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
-    // bf16 inputs at head dimension 64 or 128 run on the matrix cores, 64 steps per iteration
-    // (fp32 `out` is the recurrent_gla_naive flavour: it stays on the fp32 vector path below)
-    if (dtype == GLA_BF16 && out_dtype == GLA_BF16 && (DK == 64 || DK == 128))
-        return gla::launch_recurrent_stream_fwd<__bf16>(st, B, T, H, DK, reverse, hidden_init, log_fgate, value,
-                                                        key, query, hidden_final, out);
+    // bf16 inputs at head dimension 64 or 128 run on the matrix cores, 64 or 128 steps per iteration; fp32 `out`
+    // (the recurrent_gla_naive flavour, gla.py:37) is the same kernel storing its fp32 accumulators unrounded
+    if (dtype == GLA_BF16 && (DK == 64 || DK == 128)) {
+        if (out_dtype == GLA_F32)
+            return gla::launch_recurrent_stream_fwd<float>(st, B, T, H, DK, reverse, hidden_dtype, hidden_init,
+                                                           log_fgate, value, key, query, hidden_final, out);
+        return gla::launch_recurrent_stream_fwd<__bf16>(st, B, T, H, DK, reverse, hidden_dtype, hidden_init,
+                                                        log_fgate, value, key, query, hidden_final, out);
+    }
     if (dtype == GLA_BF16 && out_dtype == GLA_BF16)
-        return gla::launch_fwd<__bf16, __bf16>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value,
+        return gla::launch_fwd<__bf16, __bf16>(st, B, T, H, DK, DV, reverse, hidden_dtype, hidden_init, log_fgate, value,
                                                key, query, hidden_final, out);
     if (dtype == GLA_BF16)
-        return gla::launch_fwd<__bf16, float>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value,
+        return gla::launch_fwd<__bf16, float>(st, B, T, H, DK, DV, reverse, hidden_dtype, hidden_init, log_fgate, value,
                                               key, query, hidden_final, out);
-    return gla::launch_fwd<float, float>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value, key,
+    return gla::launch_fwd<float, float>(st, B, T, H, DK, DV, reverse, hidden_dtype, hidden_init, log_fgate, value, key,
                                          query, hidden_final, out);
 }
 
 extern "C" int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                                 gla_dtype dtype, gla_dtype out_dtype, int reverse,
+                                 gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
                                  const void *hidden_init, const float *log_fgate, const void *value,
                                  const void *key, const void *query, const void *hidden_final,
                                  const void *dhidden_final, const void *dout, void *dhidden_init,
                                  float *dlog_fgate, void *dvalue, void *dkey, void *dquery)
 {
-    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, out_dtype);
+    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, hidden_dtype, out_dtype);
     if (rc) return rc;
     const void *ptrs[] = {hidden_init, log_fgate, value, key, query, hidden_final, dhidden_final,
                           dout, dhidden_init, dlog_fgate, dvalue, dkey, dquery};
@@ -511,14 +520,14 @@ extern "C" int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, 
     }
     hipStream_t st = (hipStream_t)stream;
     if (dtype == GLA_BF16 && out_dtype == GLA_BF16)
-        return gla::launch_bwd<__bf16, __bf16>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value,
+        return gla::launch_bwd<__bf16, __bf16>(st, B, T, H, DK, DV, reverse, hidden_dtype, hidden_init, log_fgate, value,
                                                key, query, hidden_final, dhidden_final, dout, dhidden_init,
                                                dlog_fgate, dvalue, dkey, dquery);
     if (dtype == GLA_BF16)
-        return gla::launch_bwd<__bf16, float>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value,
+        return gla::launch_bwd<__bf16, float>(st, B, T, H, DK, DV, reverse, hidden_dtype, hidden_init, log_fgate, value,
                                               key, query, hidden_final, dhidden_final, dout, dhidden_init,
                                               dlog_fgate, dvalue, dkey, dquery);
-    return gla::launch_bwd<float, float>(st, B, T, H, DK, DV, reverse, hidden_init, log_fgate, value, key,
+    return gla::launch_bwd<float, float>(st, B, T, H, DK, DV, reverse, hidden_dtype, hidden_init, log_fgate, value, key,
                                          query, hidden_final, dhidden_final, dout, dhidden_init, dlog_fgate,
                                          dvalue, dkey, dquery);
 }

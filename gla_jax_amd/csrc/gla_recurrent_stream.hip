@@ -32,9 +32,9 @@ template <> struct OutPack<float> {
 
 template <typename TO, int C, int D>
 __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
-    const __bf16 *__restrict__ h0, const float *__restrict__ g, const __bf16 *__restrict__ v,
-    const __bf16 *__restrict__ k, const __bf16 *__restrict__ q, __bf16 *__restrict__ hT,
-    TO *__restrict__ out, int T_len, int H, int reverse)
+    const void *__restrict__ h0, const float *__restrict__ g, const __bf16 *__restrict__ v,
+    const __bf16 *__restrict__ k, const __bf16 *__restrict__ q, void *__restrict__ hT,
+    TO *__restrict__ out, int T_len, int H, int reverse, int hdt)
 {
     typedef __bf16 T;
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16;
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
             float t4[4];
-            load_vec<T, 4>(h0 + bh * D * D + (int64_t)(16 * (nt0 + nt) + r) * D + 16 * (wv + i * NDV) + 4 * c, t4);
+            load_hidden<4>(h0, hdt, bh * D * D + (int64_t)(16 * (nt0 + nt) + r) * D + 16 * (wv + i * NDV) + 4 * c, t4);
             S[i][nt] = f32x4{t4[0], t4[1], t4[2], t4[3]};
         }
     auto publish_state = [&]() {
@@ -245,12 +245,12 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
             float t4[4] = {S[i][nt][0], S[i][nt][1], S[i][nt][2], S[i][nt][3]};
-            store_vec<T, 4>(hT + bh * D * D + (int64_t)(16 * (nt0 + nt) + r) * D + 16 * (wv + i * NDV) + 4 * c, t4);
+            store_hidden<4>(hT, hdt, bh * D * D + (int64_t)(16 * (nt0 + nt) + r) * D + 16 * (wv + i * NDV) + 4 * c, t4);
         }
 }
 
 template <typename TO, int C, int D>
-static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, const void *h0, const float *g,
+static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, int hdt, const void *h0, const float *g,
                       const void *v, const void *k, const void *q, void *hT, void *out)
 {
     typedef __bf16 T;
@@ -260,25 +260,25 @@ static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, cons
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
-    hipLaunchKernelGGL(kern, grid, block, lds, st, (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,
-                       (T *)hT, (TO *)out, T_len, H, reverse);
+    hipLaunchKernelGGL(kern, grid, block, lds, st, h0, g, (const T *)v, (const T *)k, (const T *)q, hT, (TO *)out,
+                       T_len, H, reverse, hdt);
     return launch_status();
 }
 
 template <typename TO>
-int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
-                                const float *g, const void *v, const void *k, const void *q, void *hT,
-                                void *out)
+int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt,
+                                const void *h0, const float *g, const void *v, const void *k, const void *q,
+                                void *hT, void *out)
 {
-    if (D == 64) return launch_one<TO, 128, 64>(st, B, T_len, H, reverse, h0, g, v, k, q, hT, out);
-    if (D == 128) return launch_one<TO, 64, 128>(st, B, T_len, H, reverse, h0, g, v, k, q, hT, out);
+    if (D == 64) return launch_one<TO, 128, 64>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, out);
+    if (D == 128) return launch_one<TO, 64, 128>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, out);
     return GLA_ERR_UNSUPPORTED;
 }
 
-template int launch_recurrent_stream_fwd<__bf16>(hipStream_t, int, int, int, int, int, const void *,
+template int launch_recurrent_stream_fwd<__bf16>(hipStream_t, int, int, int, int, int, int, const void *,
                                                  const float *, const void *, const void *, const void *,
                                                  void *, void *);
-template int launch_recurrent_stream_fwd<float>(hipStream_t, int, int, int, int, int, const void *,
+template int launch_recurrent_stream_fwd<float>(hipStream_t, int, int, int, int, int, int, const void *,
                                                 const float *, const void *, const void *, const void *,
                                                 void *, void *);
 

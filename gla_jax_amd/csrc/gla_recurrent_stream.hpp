@@ -1,4 +1,5 @@
-// Launchers of the matrix-core recurrent_gla kernels (bf16 inputs, head dimension 64 or 128).
+// Launchers of the matrix-core recurrent_gla kernels (bf16 inputs, head dimension 64 or 128).  `hdt` is the
+// gla_dtype of the state arrays (h0, hT, dhT, dh0).
 #pragma once
 
 #include "gla_common.hpp"
@@ -7,29 +8,29 @@ namespace gla {
 
 // TO = element type of `out` (__bf16, or float for the recurrent_gla_naive flavour).
 template <typename TO>
-int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
-                                const float *g, const void *v, const void *k, const void *q, void *hT,
-                                void *out);
+int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt,
+                                const void *h0, const float *g, const void *v, const void *k, const void *q,
+                                void *hT, void *out);
 
-// Sweep 1 of the backward (bf16 everywhere): dq, and q*dq in fp32 into `qdq` (the last step's carries
-// sum_v dhT * (final state) on top).
-int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
-                               const float *g, const void *v, const void *k, const void *q, const void *dhT,
-                               const void *dout, void *dq, float *qdq);
+// Sweep 1 of the backward: dq, and q*dq in fp32 into `qdq` (the last step's carries sum_v dhT * (final state)
+// on top).  dout_f32 != 0: `dout` is float (the recurrent_gla_naive flavour), else bf16.
+int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
+                               const void *h0, const float *g, const void *v, const void *k, const void *q,
+                               const void *dhT, const void *dout, void *dq, float *qdq);
 
 // The same sweep with two waves per sub-block (head dimension 64).
-int launch_recurrent_stream_dq2(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
-                                const float *g, const void *v, const void *k, const void *q, const void *dhT,
-                                const void *dout, void *dq, float *qdq);
+int launch_recurrent_stream_dq2(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
+                                const void *h0, const float *g, const void *v, const void *k, const void *q,
+                                const void *dhT, const void *dout, void *dq, float *qdq);
 
 // Sweep 2: dk, dv, dh0 and dlog_fgate (`dg` holds sweep 1's q*dq on entry).
-int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, const float *g,
-                                const void *v, const void *k, const void *q, const void *dhT,
+int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
+                                const float *g, const void *v, const void *k, const void *q, const void *dhT,
                                 const void *dout, void *dh0, float *dg, void *dv, void *dk);
 
 // The same sweep with two waves per sub-block (head dimension 64).
-int launch_recurrent_stream_rev2(hipStream_t st, int B, int T_len, int H, int D, int reverse, const float *g,
-                                 const void *v, const void *k, const void *q, const void *dhT, const void *dout,
-                                 void *dh0, float *dg, void *dv, void *dk);
+int launch_recurrent_stream_rev2(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
+                                 const float *g, const void *v, const void *k, const void *q, const void *dhT,
+                                 const void *dout, void *dh0, float *dg, void *dv, void *dk);
 
 }  // namespace gla

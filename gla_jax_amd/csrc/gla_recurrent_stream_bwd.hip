@@ -24,11 +24,11 @@ typedef __bf16 BT;
 // ---------------------------------------------------------------------------------------------------
 // sweep 1
 // ---------------------------------------------------------------------------------------------------
-template <int C, int D>
+template <typename TO, int C, int D>
 __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
-    const BT *__restrict__ h0, const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k,
-    const BT *__restrict__ q, const BT *__restrict__ dhT, const BT *__restrict__ dout, BT *__restrict__ dq,
-    float *__restrict__ qdq, int T_len, int H, int reverse)
+    const void *__restrict__ h0, const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k,
+    const BT *__restrict__ q, const void *__restrict__ dhT, const TO *__restrict__ dout, BT *__restrict__ dq,
+    float *__restrict__ qdq, int T_len, int H, int reverse, int hdt)
 {
     typedef BT T;
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16, RT = NT / NB;
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             float t4[4];
-            load_vec<T, 4>(h0 + bh * D * D + (int64_t)(16 * nt + r) * D + 16 * (w + i * NB) + 4 * c, t4);
+            load_hidden<4>(h0, hdt, bh * D * D + (int64_t)(16 * nt + r) * D + 16 * (w + i * NB) + 4 * c, t4);
             S[i][nt] = f32x4{t4[0], t4[1], t4[2], t4[3]};
         }
     auto publish_state = [&]() {
@@ -85,7 +85,8 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
     publish_state();
 
     f32x8 gN[KS];
-    D8 qN[KS], kN[KS], vN[KS], dN[KS];
+    D8 qN[KS], kN[KS], vN[KS];
+    DoutRow<TO> dN[KS];
     bool validN;
     int64_t rowN;
     auto fetch = [&](int n) {
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
             qN[ks] = ld8(q + rowN + 32 * ks + 8 * c);
             kN[ks] = ld8(k + rowN + 32 * ks + 8 * c);
             vN[ks] = ld8(v + rowN + 32 * ks + 8 * c);
-            dN[ks] = ld8(dout + rowN + 32 * ks + 8 * c);
+            dN[ks].load(dout + rowN + 32 * ks + 8 * c);
         }
     };
     fetch(0);
@@ -119,7 +120,8 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     gN[ks] = pack8<float>(z);
-                    qN[ks] = kN[ks] = vN[ks] = dN[ks] = pack8<T>(z);
+                    qN[ks] = kN[ks] = vN[ks] = pack8<T>(z);
+                    dN[ks].zero();
                 }
             }
 #pragma unroll
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
                 qf[ks] = qN[ks];
                 kf[ks] = kN[ks];
                 vf[ks] = vN[ks];
-                dof[ks] = dN[ks];
+                dof[ks] = dN[ks].operand();
                 st8(Vn + wrow + 32 * ks, vf[ks]);
             }
 
@@ -313,12 +315,12 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
         constexpr int LPF = C * 4 / D;                                   // lanes per key feature: 4 or 2
         static_assert(LPF == 4 || LPF == 2, "a quad or a pair of lanes shares a key feature");
         const int d = threadIdx.x / LPF, part = threadIdx.x % LPF;       // each takes D / LPF of the row
-        const T *dp = dhT + bh * D * D + (int64_t)d * D + part * (D / LPF);
+        const int64_t dpo = bh * D * D + (int64_t)d * D + part * (D / LPF);
         float acc = 0.f;
 #pragma unroll
         for (int j = 0; j < D / LPF; j += 8) {
             float dv8[8], sh[8], sl[8];
-            unpack8(ld8(dp + j), dv8);
+            load_hidden<8>(dhT, hdt, dpo + j, dv8);
             unpack8(ld8(Sh + d * LS + part * (D / LPF) + j), sh);
             unpack8(ld8(Sl + d * LS + part * (D / LPF) + j), sl);
 #pragma unroll
@@ -341,11 +343,11 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
 //   dS_in = diag(e^{Lend}) dS' + sum_i (q e^{L})_i do_i^T     (a Horner chain over the sub-blocks, last first)
 // dS' is the gradient w.r.t. the state after the block.
 // ---------------------------------------------------------------------------------------------------
-template <int C, int D>
+template <typename TO, int C, int D>
 __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
     const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k, const BT *__restrict__ q,
-    const BT *__restrict__ dhT, const BT *__restrict__ dout, BT *__restrict__ dh0,
-    float *__restrict__ dg, BT *__restrict__ dv, BT *__restrict__ dk, int T_len, int H, int reverse)
+    const void *__restrict__ dhT, const TO *__restrict__ dout, void *__restrict__ dh0,
+    float *__restrict__ dg, BT *__restrict__ dv, BT *__restrict__ dk, int T_len, int H, int reverse, int hdt)
 {
     typedef BT T;
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16, RT = NT / NB;
@@ -389,7 +391,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                DS[i][nt][e] = (float)dhT[bh * D * D + (int64_t)(16 * (w + i * NB) + 4 * c + e) * D + 16 * nt + r];
+                DS[i][nt][e] = load_hidden1(dhT, hdt, bh * D * D + (int64_t)(16 * (w + i * NB) + 4 * c + e) * D + 16 * nt + r);
     auto publish = [&]() {
 #pragma unroll
         for (int i = 0; i < RT; ++i)
@@ -408,7 +410,8 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
     for (int d = threadIdx.x; d < 2 * D; d += C * 4) runtab[d] = 0.f;
 
     f32x8 gN[KS];
-    D8 qN[KS], kN[KS], vN[KS], dN[KS];
+    D8 qN[KS], kN[KS], vN[KS];
+    DoutRow<TO> dN[KS];
     bool validN;
     int64_t rowN;
     auto fetch = [&](int n) {
@@ -422,7 +425,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
             qN[ks] = ld8(q + rowN + 32 * ks + 8 * c);
             kN[ks] = ld8(k + rowN + 32 * ks + 8 * c);
             vN[ks] = ld8(v + rowN + 32 * ks + 8 * c);
-            dN[ks] = ld8(dout + rowN + 32 * ks + 8 * c);
+            dN[ks].load(dout + rowN + 32 * ks + 8 * c);
         }
     };
     fetch(N - 1);
@@ -445,7 +448,8 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     gN[ks] = pack8<float>(z);
-                    qN[ks] = kN[ks] = vN[ks] = dN[ks] = pack8<T>(z);
+                    qN[ks] = kN[ks] = vN[ks] = pack8<T>(z);
+                    dN[ks].zero();
                 }
             }
 #pragma unroll
@@ -457,7 +461,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                 qf[ks] = qN[ks];
                 kf[ks] = kN[ks];
                 vf[ks] = vN[ks];
-                dof[ks] = dN[ks];
+                dof[ks] = dN[ks].operand();
                 st8(tO + wrow + 32 * ks, dof[ks]);
             }
 #pragma unroll
@@ -752,11 +756,11 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                dh0[bh * D * D + (int64_t)(16 * (w + i * NB) + 4 * c + e) * D + 16 * nt + r] = (T)DS[i][nt][e];
+                store_hidden1(dh0, hdt, bh * D * D + (int64_t)(16 * (w + i * NB) + 4 * c + e) * D + 16 * nt + r, DS[i][nt][e]);
 }
 
-template <int C, int D>
-static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, const void *h0, const float *g,
+template <typename TO, int C, int D>
+static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, int hdt, const void *h0, const float *g,
                      const void *v, const void *k, const void *q, const void *dhT, const void *dout, void *dq,
                      float *qdq)
 {
@@ -765,17 +769,17 @@ static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, const
     constexpr int XS = 32 + 16 / (int)sizeof(T);
     const size_t lds = ((size_t)(3 * C + 2 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
                        (size_t)(C / 16) * D * sizeof(float);
-    auto kern = recurrent_stream_dq_kernel<C, D>;
+    auto kern = recurrent_stream_dq_kernel<TO, C, D>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
-    hipLaunchKernelGGL(kern, grid, block, lds, st, (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,
-                       (const T *)dhT, (const T *)dout, (T *)dq, qdq, T_len, H, reverse);
+    hipLaunchKernelGGL(kern, grid, block, lds, st, h0, g, (const T *)v, (const T *)k, (const T *)q,
+                       dhT, (const TO *)dout, (T *)dq, qdq, T_len, H, reverse, hdt);
     return launch_status();
 }
 
-template <int C, int D>
-static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, const float *g, const void *v,
+template <typename TO, int C, int D>
+static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, int hdt, const float *g, const void *v,
                       const void *k, const void *q, const void *dhT, const void *dout, void *dh0,
                       float *dg, void *dv, void *dk)
 {
@@ -784,30 +788,38 @@ static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, cons
     constexpr int XS = 32 + 16 / (int)sizeof(T);
     const size_t lds = ((size_t)(3 * C + 2 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
                        (size_t)(2 * (C / 16) + 2) * D * sizeof(float);
-    auto kern = recurrent_stream_rev_kernel<C, D>;
+    auto kern = recurrent_stream_rev_kernel<TO, C, D>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
-                       (const T *)dhT, (const T *)dout, (T *)dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse);
+                       dhT, (const TO *)dout, dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse, hdt);
     return launch_status();
 }
 
-int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, const float *g,
-                                const void *v, const void *k, const void *q, const void *dhT,
+int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
+                                const float *g, const void *v, const void *k, const void *q, const void *dhT,
                                 const void *dout, void *dh0, float *dg, void *dv, void *dk)
 {
-    if (D == 64) return launch_recurrent_stream_rev2(st, B, T_len, H, D, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
-    if (D == 128) return launch_rev<64, 128>(st, B, T_len, H, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
+    if (D == 64)
+        return launch_recurrent_stream_rev2(st, B, T_len, H, D, reverse, hdt, dout_f32, g, v, k, q, dhT, dout, dh0, dg,
+                                            dv, dk);
+    if (D == 128 && dout_f32)
+        return launch_rev<float, 64, 128>(st, B, T_len, H, reverse, hdt, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
+    if (D == 128) return launch_rev<BT, 64, 128>(st, B, T_len, H, reverse, hdt, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
     return GLA_ERR_UNSUPPORTED;
 }
 
-int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
-                               const float *g, const void *v, const void *k, const void *q, const void *dhT,
-                               const void *dout, void *dq, float *qdq)
+int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
+                               const void *h0, const float *g, const void *v, const void *k, const void *q,
+                               const void *dhT, const void *dout, void *dq, float *qdq)
 {
-    if (D == 64) return launch_recurrent_stream_dq2(st, B, T_len, H, D, reverse, h0, g, v, k, q, dhT, dout, dq, qdq);
-    if (D == 128) return launch_dq<64, 128>(st, B, T_len, H, reverse, h0, g, v, k, q, dhT, dout, dq, qdq);
+    if (D == 64)
+        return launch_recurrent_stream_dq2(st, B, T_len, H, D, reverse, hdt, dout_f32, h0, g, v, k, q, dhT, dout, dq,
+                                           qdq);
+    if (D == 128 && dout_f32)
+        return launch_dq<float, 64, 128>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, dhT, dout, dq, qdq);
+    if (D == 128) return launch_dq<BT, 64, 128>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, dhT, dout, dq, qdq);
     return GLA_ERR_UNSUPPORTED;
 }
 

@@ -9,6 +9,25 @@ namespace gla {
 
 typedef __bf16 BT;
 
+// Eight consecutive elements of a `dout` row on their way from memory to the bf16 tile the products read.  TO is
+// the element type of `dout`: bf16 for recurrent_gla; float for the recurrent_gla_naive flavour, whose `out` is
+// fp32 (gla.py:37) and so is its cotangent.  There the row is rounded to bf16 where it enters the tile (every
+// gradient it feeds is stored in bf16 or is a sum over many steps, so the 2^-9 of that rounding stays below the
+// storage rounding of the results).
+template <typename TO> struct DoutRow;
+template <> struct DoutRow<BT> {
+    bf16x8 raw;
+    __device__ __forceinline__ void load(const BT *p) { raw = ld8(p); }
+    __device__ __forceinline__ void zero() { const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; raw = pack8<BT>(z); }
+    __device__ __forceinline__ bf16x8 operand() const { return raw; }
+};
+template <> struct DoutRow<float> {
+    f32x8 raw;
+    __device__ __forceinline__ void load(const float *p) { raw = ld8(p); }
+    __device__ __forceinline__ void zero() { const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; raw = pack8<float>(z); }
+    __device__ __forceinline__ bf16x8 operand() const { return pack8<BT>(raw.v); }
+};
+
 // One level (half-width H) of the dyadic recursion of a 16-token sub-block on a 32-feature slice: the mixed
 // tile X (upper rows q e^{prefix}, lower rows k e^{suffix}) goes through the wave's scratch, dX = (M + M^T) X
 // with M the level's masked dA block; adds the query part (upper rows) to dq8 and/or the key part (lower

@@ -21,11 +21,11 @@ namespace gla {
 // ---------------------------------------------------------------------------------------------------
 // sweep 1: dq and q*dq, the state S in accumulator registers
 // ---------------------------------------------------------------------------------------------------
-template <int C, int D>
+template <typename TO, int C, int D>
 __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
-    const BT *__restrict__ h0, const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k,
-    const BT *__restrict__ q, const BT *__restrict__ dhT, const BT *__restrict__ dout, BT *__restrict__ dq,
-    float *__restrict__ qdq, int T_len, int H, int reverse)
+    const void *__restrict__ h0, const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k,
+    const BT *__restrict__ q, const void *__restrict__ dhT, const TO *__restrict__ dout, BT *__restrict__ dq,
+    float *__restrict__ qdq, int T_len, int H, int reverse, int hdt)
 {
     typedef BT T;
     constexpr int NB = C / 16, NW = 2 * NB, KS = D / 32, NT = D / 16;
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         float t4[4];
-        load_vec<T, 4>(h0 + bh * D * D + (int64_t)(16 * (nt0 + j) + r) * D + 16 * tv + 4 * c, t4);
+        load_hidden<4>(h0, hdt, bh * D * D + (int64_t)(16 * (nt0 + j) + r) * D + 16 * tv + 4 * c, t4);
         S[j] = f32x4{t4[0], t4[1], t4[2], t4[3]};
     }
     auto publish_state = [&]() {
@@ -85,7 +85,8 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
     publish_state();
 
     f32x8 gN;
-    D8 qN, kN, vN, dN;
+    D8 qN, kN, vN;
+    DoutRow<TO> dN;
     bool validN;
     int64_t rowN;
     // The rows of a block are requested in three pieces (gates; q, k; v, dout), see the loop.
@@ -102,7 +103,7 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
     };
     auto fetch_vo = [&]() {
         vN = ld8(v + rowN);
-        dN = ld8(dout + rowN);
+        dN.load(dout + rowN);
     };
     fetch_g(0);
     fetch_qk();
@@ -139,14 +140,15 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
             if ((n + 1) * C > T_len && !valid) {   // only the last block can hold padded steps
                 float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 gN = pack8<float>(z);
-                qN = kN = vN = dN = pack8<T>(z);
+                qN = kN = vN = pack8<T>(z);
+                dN.zero();
             }
 #pragma unroll
             for (int e = 0; e < 8; ++e) p[e] = gN.v[e] * kLog2e;
             qf = qN;
             unpack8(kN, bq);
             st8(Vn + wrow + fo, vN);
-            st8(tO + wrow + fo, dN);
+            st8(tO + wrow + fo, dN.operand());
 
             // gate prefix, totals through the wave's half of the table row, one anchor or not
             float *rt = rtab + I * D + fo + 8 * c;
@@ -367,7 +369,7 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
         static_assert(LPF == 8, "eight neighbouring lanes share a key feature");
         const int d = threadIdx.x / LPF, part = threadIdx.x % LPF;       // each takes D / LPF = 8 of the row
         float dv8[8], sh[8], sl[8], acc = 0.f;
-        unpack8(ld8(dhT + bh * D * D + (int64_t)d * D + part * 8), dv8);
+        load_hidden<8>(dhT, hdt, bh * D * D + (int64_t)d * D + part * 8, dv8);
         unpack8(ld8(Sh + d * LS + part * 8), sh);
         unpack8(ld8(Sl + d * LS + part * 8), sl);
 #pragma unroll
@@ -382,8 +384,8 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
     }
 }
 
-template <int C, int D>
-static int launch_dq2(hipStream_t st, int B, int T_len, int H, int reverse, const void *h0, const float *g,
+template <typename TO, int C, int D>
+static int launch_dq2(hipStream_t st, int B, int T_len, int H, int reverse, int hdt, const void *h0, const float *g,
                       const void *v, const void *k, const void *q, const void *dhT, const void *dout, void *dq,
                       float *qdq)
 {
@@ -392,12 +394,12 @@ static int launch_dq2(hipStream_t st, int B, int T_len, int H, int reverse, cons
     constexpr int XS = 32 + 16 / (int)sizeof(T);
     const size_t lds = ((size_t)(4 * C + 2 * D) * LS + (size_t)(C / 8) * 2 * 16 * XS) * sizeof(T) +
                        (size_t)(C / 16) * D * sizeof(float);
-    auto kern = recurrent_stream_dq2_kernel<C, D>;
+    auto kern = recurrent_stream_dq2_kernel<TO, C, D>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 8);
-    hipLaunchKernelGGL(kern, grid, block, lds, st, (const T *)h0, g, (const T *)v, (const T *)k, (const T *)q,
-                       (const T *)dhT, (const T *)dout, (T *)dq, qdq, T_len, H, reverse);
+    hipLaunchKernelGGL(kern, grid, block, lds, st, h0, g, (const T *)v, (const T *)k, (const T *)q,
+                       dhT, (const TO *)dout, (T *)dq, qdq, T_len, H, reverse, hdt);
     return launch_status();
 }
 
@@ -407,11 +409,11 @@ static int launch_dq2(hipStream_t st, int B, int T_len, int H, int reverse, cons
 // features fo.. for dv.  The scores A = Q~ K~^T contract over the key features: each wave forms them on its
 // slice and the two waves of a sub-block add their halves through LDS (one more barrier per block).
 // ---------------------------------------------------------------------------------------------------
-template <int C, int D>
+template <typename TO, int C, int D>
 __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
     const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k, const BT *__restrict__ q,
-    const BT *__restrict__ dhT, const BT *__restrict__ dout, BT *__restrict__ dh0,
-    float *__restrict__ dg, BT *__restrict__ dv, BT *__restrict__ dk, int T_len, int H, int reverse)
+    const void *__restrict__ dhT, const TO *__restrict__ dout, void *__restrict__ dh0,
+    float *__restrict__ dg, BT *__restrict__ dv, BT *__restrict__ dk, int T_len, int H, int reverse, int hdt)
 {
     typedef BT T;
     constexpr int NB = C / 16, NW = 2 * NB, KS = D / 32, NT = D / 16;
@@ -462,7 +464,7 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            DS[j][e] = (float)dhT[bh * D * D + (int64_t)(16 * td + 4 * c + e) * D + 16 * (nt0 + j) + r];
+            DS[j][e] = load_hidden1(dhT, hdt, bh * D * D + (int64_t)(16 * td + 4 * c + e) * D + 16 * (nt0 + j) + r);
     auto publish = [&]() {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -479,7 +481,8 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
     // Memory traffic is spread over the block as in sweep 1: the next block's rows are requested in four pieces
     // (gates; q, k; sweep 1's q*dq; v, dout) and a block's results are stored one block late, in three pieces.
     f32x8 gN, qdqN;
-    D8 qN, kN, vN, dN;
+    D8 qN, kN, vN;
+    DoutRow<TO> dN;
     bool validN;
     int64_t rowN;
     auto fetch_g = [&](int n) {
@@ -496,7 +499,7 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
     auto fetch_qdq = [&]() { qdqN = ld8(dg + rowN); };
     auto fetch_vo = [&]() {
         vN = ld8(v + rowN);
-        dN = ld8(dout + rowN);
+        dN.load(dout + rowN);
     };
     fetch_g(N - 1);
     fetch_qk();
@@ -517,7 +520,8 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
             if ((n + 1) * C > T_len && !valid) {   // only the last block can hold padded steps
                 float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 gN = pack8<float>(z);
-                qN = kN = vN = dN = pack8<T>(z);
+                qN = kN = vN = pack8<T>(z);
+                dN.zero();
             }
 #pragma unroll
             for (int e = 0; e < 8; ++e) p[e] = gN.v[e] * kLog2e;
@@ -527,7 +531,7 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
                 float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 qdqN = pack8<float>(z);
             }
-            st8(tO + wrow + fo, dN);
+            st8(tO + wrow + fo, dN.operand());
             st8(Vn + wrow + fo, vN);
 
             float *rt = rtab + J0 * D + fo + 8 * c;
@@ -837,11 +841,11 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            dh0[bh * D * D + (int64_t)(16 * td + 4 * c + e) * D + 16 * (nt0 + j) + r] = (T)DS[j][e];
+            store_hidden1(dh0, hdt, bh * D * D + (int64_t)(16 * td + 4 * c + e) * D + 16 * (nt0 + j) + r, DS[j][e]);
 }
 
-template <int C, int D>
-static int launch_rev2(hipStream_t st, int B, int T_len, int H, int reverse, const float *g, const void *v,
+template <typename TO, int C, int D>
+static int launch_rev2(hipStream_t st, int B, int T_len, int H, int reverse, int hdt, const float *g, const void *v,
                        const void *k, const void *q, const void *dhT, const void *dout, void *dh0, float *dg,
                        void *dv, void *dk)
 {
@@ -851,28 +855,32 @@ static int launch_rev2(hipStream_t st, int B, int T_len, int H, int reverse, con
     constexpr int NB = C / 16, NW = 2 * NB;
     const size_t lds = ((size_t)(6 * C + 2 * D) * LS + (size_t)NW * 2 * 16 * XS) * sizeof(T) +
                        (size_t)(2 * NB + 2) * D * sizeof(float) + (size_t)NW * NB * 64 * sizeof(f32x4);
-    auto kern = recurrent_stream_rev2_kernel<C, D>;
+    auto kern = recurrent_stream_rev2_kernel<TO, C, D>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 8);
-    hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q, (const T *)dhT,
-                       (const T *)dout, (T *)dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse);
+    hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q, dhT,
+                       (const TO *)dout, dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse, hdt);
     return launch_status();
 }
 
-int launch_recurrent_stream_rev2(hipStream_t st, int B, int T_len, int H, int D, int reverse, const float *g,
-                                 const void *v, const void *k, const void *q, const void *dhT, const void *dout,
-                                 void *dh0, float *dg, void *dv, void *dk)
+int launch_recurrent_stream_rev2(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
+                                 const float *g, const void *v, const void *k, const void *q, const void *dhT,
+                                 const void *dout, void *dh0, float *dg, void *dv, void *dk)
 {
-    if (D == 64) return launch_rev2<64, 64>(st, B, T_len, H, reverse, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
+    if (D == 64 && dout_f32)
+        return launch_rev2<float, 64, 64>(st, B, T_len, H, reverse, hdt, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
+    if (D == 64) return launch_rev2<BT, 64, 64>(st, B, T_len, H, reverse, hdt, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
     return GLA_ERR_UNSUPPORTED;
 }
 
-int launch_recurrent_stream_dq2(hipStream_t st, int B, int T_len, int H, int D, int reverse, const void *h0,
-                                const float *g, const void *v, const void *k, const void *q, const void *dhT,
-                                const void *dout, void *dq, float *qdq)
+int launch_recurrent_stream_dq2(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
+                                const void *h0, const float *g, const void *v, const void *k, const void *q,
+                                const void *dhT, const void *dout, void *dq, float *qdq)
 {
-    if (D == 64) return launch_dq2<64, 64>(st, B, T_len, H, reverse, h0, g, v, k, q, dhT, dout, dq, qdq);
+    if (D == 64 && dout_f32)
+        return launch_dq2<float, 64, 64>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, dhT, dout, dq, qdq);
+    if (D == 64) return launch_dq2<BT, 64, 64>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, dhT, dout, dq, qdq);
     return GLA_ERR_UNSUPPORTED;
 }
 

@@ -30,8 +30,8 @@ def _ptr(t):
 
 def _prep(hidden_init, log_fgate, value, key, query):
     """Checks the reference's shape contract and returns the canonical 4-D views the kernels take
-    (h0 [B,H,DK,DV], g/k/q [B,T,H,DK], v [B,T,H,DV]; dense, gates fp32, hidden in the value dtype), the
-    leading batch shape and the dims.  Everything here is a differentiable torch op (reshape, cast, copy),
+    (h0 [B,H,DK,DV], g/k/q [B,T,H,DK], v [B,T,H,DV]; dense, gates fp32, hidden in its own dtype when that is
+    float32 or bfloat16, else in float32), the leading batch shape and the dims.  Everything here is a differentiable torch op (reshape, cast, copy),
     so autograd carries gradients back to the caller's own layouts and dtypes; for arrays that are
     already dense and typed as the kernels want them nothing is copied."""
     for name, t in (("hidden_init", hidden_init), ("log_fgate", log_fgate), ("value", value),
@@ -59,9 +59,10 @@ def _prep(hidden_init, log_fgate, value, key, query):
     B = 1
     for s in lead:
         B *= s
-    # the state enters the kernels in the value dtype (the reference's chunk path casts it the same way,
-    # gla.py:720) and hidden_final goes back out in hidden_init's own dtype (gla.py:46, 727)
-    h0 = _as(hidden_init, (B, H, DK, DV), dt)
+    # the state enters the kernels in its own dtype: the reference loads it uncast into an fp32 state
+    # (gla.py:44, 89; the chunk scan takes it uncast too, gla.py:711-716) and stores hidden_final back in
+    # hidden_init's dtype (gla.py:46, 97, 727).  Other float types (half, double) go through float32.
+    h0 = _as(hidden_init, (B, H, DK, DV), hidden_init.dtype if hidden_init.dtype in _DT else torch.float32)
     g = _as(log_fgate, (B, T, H, DK), torch.float32)                       # gates are fp32 (gla.py:495)
     v = _as(value, (B, T, H, DV), dt)
     k = _as(key, (B, T, H, DK), dt)
@@ -147,7 +148,7 @@ def _chunk_forward(h0, g, v, k, q, chunk_size, residual):
     states = torch.empty(st_bytes, dtype=torch.uint8, device=v.device) if residual else None
     hT = torch.empty_like(h0)
     out = torch.empty_like(v)
-    rc = lib.gla_chunk_fwd(_stream(), B, T, H, DK, DV, chunk_size, dt, _ptr(h0), _ptr(g), _ptr(v),
+    rc = lib.gla_chunk_fwd(_stream(), B, T, H, DK, DV, chunk_size, dt, _DT[h0.dtype], _ptr(h0), _ptr(g), _ptr(v),
                            _ptr(k), _ptr(q), _ptr(hT), _ptr(out), _ptr(states), _ptr(ws), ws_bytes)
     _lib.check("gla_chunk_fwd", rc)
     return hT, out, states
@@ -167,6 +168,7 @@ class _ChunkGLA(torch.autograd.Function):
         states = output[2]
         ctx.save_for_backward(states, g, v, k, q)          # residuals of gla.py:542-549
         ctx.chunk_size = chunk_size
+        ctx.hidden_dtype = h0.dtype
         ctx.mark_non_differentiable(states)
 
     @staticmethod
@@ -174,7 +176,7 @@ class _ChunkGLA(torch.autograd.Function):
         states, g, v, k, q = ctx.saved_tensors
         B, T, H, DK = k.shape
         DV = v.shape[-1]
-        dhT = torch.zeros(B, H, DK, DV, dtype=v.dtype, device=v.device) if dhT is None else dhT
+        dhT = torch.zeros(B, H, DK, DV, dtype=ctx.hidden_dtype, device=v.device) if dhT is None else dhT
         dout = torch.zeros_like(v) if dout is None else dout
         return _apply(_ChunkGLABwd, states, g, v, k, q, dhT, dout, ctx.chunk_size) + (None,)
 
@@ -196,14 +198,15 @@ class _ChunkGLABwd(torch.autograd.Function):
         DV = v.shape[-1]
         lib = _lib.load()
         dt = _DT[v.dtype]
-        dhT = dhT.to(v.dtype).contiguous()
+        # the cotangent of hidden_final arrives in the state's dtype; dhidden_init goes back in it
+        dhT = dhT.to(dhT.dtype if dhT.dtype in _DT else torch.float32).contiguous()
         dout = dout.to(v.dtype).contiguous()
         ws_bytes = lib.gla_chunk_bwd_workspace_bytes(B, T, H, DK, DV, chunk_size, dt)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=v.device)
         dh0 = torch.empty_like(dhT)
         dg = torch.empty_like(g)
         dv, dk, dq = torch.empty_like(v), torch.empty_like(k), torch.empty_like(q)
-        rc = lib.gla_chunk_bwd(_stream(), B, T, H, DK, DV, chunk_size, dt, _ptr(g), _ptr(v), _ptr(k),
+        rc = lib.gla_chunk_bwd(_stream(), B, T, H, DK, DV, chunk_size, dt, _DT[dhT.dtype], _ptr(g), _ptr(v), _ptr(k),
                                _ptr(q), _ptr(states), _ptr(dhT), _ptr(dout), _ptr(dh0), _ptr(dg),
                                _ptr(dv), _ptr(dk), _ptr(dq), _ptr(ws), ws_bytes)
         _lib.check("gla_chunk_bwd", rc)
@@ -268,7 +271,7 @@ class _RecurrentGLA(torch.autograd.Function):
         odt = _lib.GLA_F32 if out_fp32 else dt
         hT = torch.empty_like(h0)
         out = torch.empty(v.shape, dtype=torch.float32 if out_fp32 else v.dtype, device=v.device)
-        rc = lib.gla_recurrent_fwd(_stream(), B, T, H, DK, DV, dt, odt, int(bool(reverse)), _ptr(h0),
+        rc = lib.gla_recurrent_fwd(_stream(), B, T, H, DK, DV, dt, _DT[h0.dtype], odt, int(bool(reverse)), _ptr(h0),
                                    _ptr(g), _ptr(v), _ptr(k), _ptr(q), _ptr(hT), _ptr(out))
         _lib.check("gla_recurrent_fwd", rc)
         return hT, out
@@ -305,13 +308,14 @@ class _RecurrentGLABwd(torch.autograd.Function):
         lib = _lib.load()
         dt = _DT[v.dtype]
         odt = _lib.GLA_F32 if out_fp32 else dt
-        dhT = dhT.to(v.dtype).contiguous()
+        dhT = dhT.to(h0.dtype).contiguous()                # the four state arrays share hidden_init's dtype
         dout = dout.to(torch.float32 if out_fp32 else v.dtype).contiguous()
-        hTc = hT.contiguous()
+        hTc = hT.to(h0.dtype).contiguous()
         dh0 = torch.empty_like(h0)
         dg = torch.empty_like(g)
         dv, dk, dq = torch.empty_like(v), torch.empty_like(k), torch.empty_like(q)
-        rc = lib.gla_recurrent_bwd(_stream(), B, T, H, DK, DV, dt, odt, int(bool(reverse)), _ptr(h0), _ptr(g),
+        rc = lib.gla_recurrent_bwd(_stream(), B, T, H, DK, DV, dt, _DT[h0.dtype], odt, int(bool(reverse)), _ptr(h0),
+                                   _ptr(g),
                                    _ptr(v), _ptr(k), _ptr(q), _ptr(hTc), _ptr(dhT), _ptr(dout),
                                    _ptr(dh0), _ptr(dg), _ptr(dv), _ptr(dk), _ptr(dq))
         _lib.check("gla_recurrent_bwd", rc)

@@ -65,6 +65,13 @@ def _like(x, dtype=None):
     return jax.ShapeDtypeStruct(x.shape, x.dtype if dtype is None else dtype)
 
 
+def _state(hidden):
+    """The state as the kernels take it: in its own dtype when that is float32 or bfloat16 (the reference loads
+    hidden_init uncast into an fp32 state, gla.py:44, 89, and hands it uncast to the chunk scan, gla.py:711-716),
+    through float32 otherwise."""
+    return hidden if hidden.dtype in (jnp.float32, jnp.bfloat16) else hidden.astype(jnp.float32)
+
+
 # ---------------------------------------------------------------------------------------------- chunk_gla
 @functools.partial(jax.custom_vjp, nondiff_argnums=(5,))
 def chunk_gla_forward_backward(hidden_init, log_fgate, value, key, query, chunk_size):      # gla.py:628-655
@@ -73,7 +80,7 @@ def chunk_gla_forward_backward(hidden_init, log_fgate, value, key, query, chunk_
 
 def _chunk_fwd(hidden_init, log_fgate, value, key, query, chunk_size):
     st, wf, _ = _sizes(key, value, chunk_size)
-    h0 = hidden_init.astype(value.dtype)
+    h0 = _state(hidden_init)
     g = log_fgate.astype(jnp.float32)
     hT, out, states, _ws = jax.ffi.ffi_call(
         "GlaChunkFwd",
@@ -88,9 +95,9 @@ def _chunk_bwd(chunk_size, res, cotangents):
     _, _, wb = _sizes(key, value, chunk_size)
     dh0, dg, dv, dk, dq, _ws = jax.ffi.ffi_call(
         "GlaChunkBwd",
-        (_like(dhT, value.dtype), _like(g), _like(value), _like(key), _like(query),
+        (_like(_state(dhT)), _like(g), _like(value), _like(key), _like(query),
          jax.ShapeDtypeStruct((wb,), jnp.uint8)),
-        vmap_method="broadcast_all")(g, value, key, query, states, dhT.astype(value.dtype),
+        vmap_method="broadcast_all")(g, value, key, query, states, _state(dhT),
                                      dout.astype(value.dtype), chunk_size=int(chunk_size))
     return dh0.astype(h_dtype), dg.astype(g_dtype), dv, dk, dq                                 # gla.py:625
 
@@ -117,7 +124,7 @@ def recurrent_gla_forward_backward(hidden_init, log_fgate, value, key, query, re
 
 
 def _rec_fwd(hidden_init, log_fgate, value, key, query, reverse, out_fp32):
-    h0 = hidden_init.astype(value.dtype)
+    h0 = _state(hidden_init)
     g = log_fgate.astype(jnp.float32)
     hT, out = jax.ffi.ffi_call(
         "GlaRecurrentFwd", (_like(h0), _like(value, jnp.float32 if out_fp32 else None)),
@@ -131,7 +138,7 @@ def _rec_bwd(reverse, out_fp32, res, cotangents):
     dhT, dout = cotangents
     dh0, dg, dv, dk, dq = jax.ffi.ffi_call(
         "GlaRecurrentBwd", (_like(h0), _like(g), _like(value), _like(key), _like(query)),
-        vmap_method="broadcast_all")(h0, g, value, key, query, hT, dhT.astype(value.dtype),
+        vmap_method="broadcast_all")(h0, g, value, key, query, hT, dhT.astype(h0.dtype),
                                      dout.astype(jnp.float32 if out_fp32 else value.dtype),
                                      reverse=bool(reverse))
     return dh0.astype(h_dtype), dg.astype(g_dtype), dv, dk, dq                                   # gla.py:269
@@ -165,11 +172,17 @@ def cumsum_recursive(src, axis, init=None, reverse=False, block_size_t=2048):
     return out.astype(src.dtype)
 
 
-def rnn_recursive(log_fgate, kv, init_log_fgate, init_kv, reverse=False, block_size_t=256):
-    """ops.py:396-456: x_n = exp(a_n)[:,None] * x_{n-1} + b_n with init (reverse: from the far end); returns
-    (running sum of a including its init, states).  fp32 arithmetic, results in the input dtypes."""
+def rnn_recursive(log_fgate, kv, init_log_fgate=None, init_kv=None, block_size_t=256, reverse=False):
+    """ops.py:396-456: x_n = exp(a_n)[:,None] * x_{n-1} + b_n with an optional initial pair (reverse: from the
+    far end); returns (running sum of a including its init, states).  fp32 arithmetic, results in the input
+    dtypes.  `block_size_t` is the reference's recursion knob and has no effect."""
+    assert (init_log_fgate is None) == (init_kv is None), "init_log_fgate and init_kv go together"   # ops.py:407
     a, b = log_fgate.astype(jnp.float32), kv.astype(jnp.float32)
-    ia, ib = init_log_fgate.astype(jnp.float32), init_kv.astype(jnp.float32)
+    if init_kv is None:                      # the reference starts from a zero gate sum and a zero state
+        ia = jnp.zeros(a.shape[:-2] + a.shape[-1:], jnp.float32)
+        ib = jnp.zeros(b.shape[:-3] + b.shape[-2:], jnp.float32)
+    else:
+        ia, ib = init_log_fgate.astype(jnp.float32), init_kv.astype(jnp.float32)
     oa, ob = jax.ffi.ffi_call("GlaRnnScan", (_like(a), _like(b)), vmap_method="broadcast_all")(
         a, b, ia, ib, reverse=bool(reverse))
     return oa.astype(log_fgate.dtype), ob.astype(kv.dtype)

@@ -73,10 +73,12 @@ ffi::Error ChunkFwd(hipStream_t stream, int64_t chunk_size, ffi::AnyBuffer h0, f
                     ffi::Result<ffi::AnyBuffer> workspace)
 {
     Dims d = dims_of(k, v);
-    gla_dtype dt;
-    if (!d.ok || !dtype_of(v.element_type(), &dt)) return ffi::Error::InvalidArgument("gla_chunk_fwd: bad operands");
+    gla_dtype dt, hdt;                       // the state arrays carry a dtype of their own (gla.py:711-716, 727)
+    if (!d.ok || !dtype_of(v.element_type(), &dt) || !dtype_of(h0.element_type(), &hdt) ||
+        hT->element_type() != h0.element_type())
+        return ffi::Error::InvalidArgument("gla_chunk_fwd: bad operands");
     return status("gla_chunk_fwd",
-                  gla_chunk_fwd(stream, d.B, d.T, d.H, d.DK, d.DV, chunk_size, dt, h0.untyped_data(),
+                  gla_chunk_fwd(stream, d.B, d.T, d.H, d.DK, d.DV, chunk_size, dt, hdt, h0.untyped_data(),
                                 g.typed_data(), v.untyped_data(), k.untyped_data(), q.untyped_data(),
                                 hT->untyped_data(), out->untyped_data(), states->untyped_data(),
                                 workspace->untyped_data(), workspace->size_bytes()));
@@ -91,10 +93,12 @@ ffi::Error ChunkBwd(hipStream_t stream, int64_t chunk_size, ffi::Buffer<ffi::F32
                     ffi::Result<ffi::AnyBuffer> dq, ffi::Result<ffi::AnyBuffer> workspace)
 {
     Dims d = dims_of(k, v);
-    gla_dtype dt;
-    if (!d.ok || !dtype_of(v.element_type(), &dt)) return ffi::Error::InvalidArgument("gla_chunk_bwd: bad operands");
+    gla_dtype dt, hdt;
+    if (!d.ok || !dtype_of(v.element_type(), &dt) || !dtype_of(dhT.element_type(), &hdt) ||
+        dh0->element_type() != dhT.element_type())
+        return ffi::Error::InvalidArgument("gla_chunk_bwd: bad operands");
     return status("gla_chunk_bwd",
-                  gla_chunk_bwd(stream, d.B, d.T, d.H, d.DK, d.DV, chunk_size, dt, g.typed_data(),
+                  gla_chunk_bwd(stream, d.B, d.T, d.H, d.DK, d.DV, chunk_size, dt, hdt, g.typed_data(),
                                 v.untyped_data(), k.untyped_data(), q.untyped_data(), states.untyped_data(),
                                 dhT.untyped_data(), dout.untyped_data(), dh0->untyped_data(), dg->typed_data(),
                                 dv->untyped_data(), dk->untyped_data(), dq->untyped_data(),
@@ -109,11 +113,12 @@ ffi::Error RecurrentFwd(hipStream_t stream, bool reverse, ffi::AnyBuffer h0, ffi
                         ffi::Result<ffi::AnyBuffer> out)
 {
     Dims d = dims_of(k, v);
-    gla_dtype dt, odt;
-    if (!d.ok || !dtype_of(v.element_type(), &dt) || !dtype_of(out->element_type(), &odt))
+    gla_dtype dt, hdt, odt;
+    if (!d.ok || !dtype_of(v.element_type(), &dt) || !dtype_of(out->element_type(), &odt) ||
+        !dtype_of(h0.element_type(), &hdt) || hT->element_type() != h0.element_type())
         return ffi::Error::InvalidArgument("gla_recurrent_fwd: bad operands");
     return status("gla_recurrent_fwd",
-                  gla_recurrent_fwd(stream, d.B, d.T, d.H, d.DK, d.DV, dt, odt, reverse ? 1 : 0,
+                  gla_recurrent_fwd(stream, d.B, d.T, d.H, d.DK, d.DV, dt, hdt, odt, reverse ? 1 : 0,
                                     h0.untyped_data(), g.typed_data(), v.untyped_data(), k.untyped_data(),
                                     q.untyped_data(), hT->untyped_data(), out->untyped_data()));
 }
@@ -126,11 +131,13 @@ ffi::Error RecurrentBwd(hipStream_t stream, bool reverse, ffi::AnyBuffer h0, ffi
                         ffi::Result<ffi::AnyBuffer> dk, ffi::Result<ffi::AnyBuffer> dq)
 {
     Dims d = dims_of(k, v);
-    gla_dtype dt, odt;
-    if (!d.ok || !dtype_of(v.element_type(), &dt) || !dtype_of(dout.element_type(), &odt))
+    gla_dtype dt, hdt, odt;
+    if (!d.ok || !dtype_of(v.element_type(), &dt) || !dtype_of(dout.element_type(), &odt) ||
+        !dtype_of(h0.element_type(), &hdt) || hT.element_type() != h0.element_type() ||
+        dhT.element_type() != h0.element_type() || dh0->element_type() != h0.element_type())
         return ffi::Error::InvalidArgument("gla_recurrent_bwd: bad operands");
     return status("gla_recurrent_bwd",
-                  gla_recurrent_bwd(stream, d.B, d.T, d.H, d.DK, d.DV, dt, odt, reverse ? 1 : 0,
+                  gla_recurrent_bwd(stream, d.B, d.T, d.H, d.DK, d.DV, dt, hdt, odt, reverse ? 1 : 0,
                                     h0.untyped_data(), g.typed_data(), v.untyped_data(), k.untyped_data(),
                                     q.untyped_data(), hT.untyped_data(), dhT.untyped_data(), dout.untyped_data(),
                                     dh0->untyped_data(), dg->typed_data(), dv->untyped_data(),

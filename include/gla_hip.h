@@ -12,8 +12,13 @@
  *       log_fgate/key/query  [B, T, H, DK]     value/out/dout  [B, T, H, DV]
  *       hidden_*             [B, H, DK, DV]
  *     log_fgate and its gradient are always float32 (gla.py:495 intent); `dtype` is the element
- *     type of hidden/value/key/query and of every output that mirrors them (out.dtype ==
- *     value.dtype gla.py:538, hidden_final.dtype == hidden_init.dtype gla.py:727).
+ *     type of value/key/query and of every output that mirrors them (out.dtype == value.dtype,
+ *     gla.py:538); `hidden_dtype` is the element type of the four state arrays hidden_init,
+ *     hidden_final, dhidden_final and dhidden_init, whatever `dtype` is: the reference loads
+ *     hidden_init in its own dtype into an fp32 state and stores hidden_final back in it
+ *     (gla.py:44-46, 89-97, 727), and hands it uncast to the chunk scan (gla.py:711-716), so an
+ *     fp32 state carried from one segment of a sequence to the next next to bf16 value/key/query
+ *     is not rounded at the hand-over.
  *   - The library never allocates, frees or synchronises: outputs and workspaces are the caller's.
  *   - Return value: 0 = enqueued; < 0 = argument rejected on the host before any launch (see
  *     gla_status); > 0 = a hipError_t from a launch.  No C++ exception crosses the boundary.
@@ -31,7 +36,7 @@
 extern "C" {
 #endif
 
-#define GLA_HIP_ABI_VERSION 1
+#define GLA_HIP_ABI_VERSION 2
 
 typedef enum gla_dtype {
     GLA_F32 = 0,
@@ -85,7 +90,7 @@ int gla_rnn_scan_f32(void *stream, const float *log_fgate, const float *kv,
  * GLA_F32 for the recurrent_gla_naive flavour whose output is fp32 by promotion, gla.py:37).
  * Requires DK == DV (gla.py:120) in {16, 32, 64, 128, 256}. */
 int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                      gla_dtype dtype, gla_dtype out_dtype, int reverse,
+                      gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
                       const void *hidden_init, const float *log_fgate, const void *value,
                       const void *key, const void *query,
                       void *hidden_final, void *out);
@@ -98,7 +103,7 @@ int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK,
  * dlog_fgate doubles as the fp32 scratch that carries q*dq from sweep 1 to sweep 2, so no workspace is
  * needed.  dout has element type out_dtype. */
 int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                      gla_dtype dtype, gla_dtype out_dtype, int reverse,
+                      gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
                       const void *hidden_init, const float *log_fgate, const void *value,
                       const void *key, const void *query, const void *hidden_final,
                       const void *dhidden_final, const void *dout,
@@ -123,9 +128,11 @@ size_t gla_chunk_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK
  * (ops.py:234), compute_intra_contrib (gla.py:792-855) with compute_score (gla.py:964-1029),
  * compute_inter_contrib (gla.py:695-729) and the chunk state scan (ops.py:396).  Requires
  * DK == DV (gla.py:499), T % chunk_size == 0, chunk_size a power of two >= 32.  `states` receives the
- * residual for the backward; pass NULL when no gradient will be taken. */
+ * residual for the backward; pass NULL when no gradient will be taken.  hidden_init enters the fp32 scan
+ * in hidden_dtype (gla.py:711-716); only its copy as the first chunk's incoming state is stored in `dtype`
+ * like every other chunk state (gla.py:719-720). */
 int gla_chunk_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                  int64_t chunk_size, gla_dtype dtype,
+                  int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
                   const void *hidden_init, const float *log_fgate, const void *value,
                   const void *key, const void *query,
                   void *hidden_final, void *out, void *states,
@@ -136,7 +143,7 @@ int gla_chunk_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int
  * compute_inter_contrib_backward gla.py:731-790, the reverse state scan and the reverse cumsum
  * gla.py:616-617).  Gradients come back in argument order (gla.py:625). */
 int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                  int64_t chunk_size, gla_dtype dtype,
+                  int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
                   const float *log_fgate, const void *value, const void *key, const void *query,
                   const void *states, const void *dhidden_final, const void *dout,
                   void *dhidden_init, float *dlog_fgate, void *dvalue, void *dkey, void *dquery,
@@ -155,7 +162,7 @@ int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int
  * in order on one stream are safe, nothing in the array has to survive from one call to the next. */
 #define GLA_CHUNK_FWD_STATIC_BYTES ((size_t)80 << 20)
 int gla_chunk_fwd_static(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                         int64_t chunk_size, gla_dtype dtype,
+                         int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
                          const void *hidden_init, const float *log_fgate, const void *value,
                          const void *key, const void *query,
                          void *hidden_final, void *out, void *states);
@@ -166,13 +173,13 @@ int gla_chunk_fwd_static(void *stream, int64_t B, int64_t T, int64_t H, int64_t 
  * the same arguments.  No counterpart in the reference; exists so that a caller can time one kernel
  * with events on its own stream (bench.py does). */
 int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                         int64_t chunk_size, gla_dtype dtype,
+                         int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
                          const void *hidden_init, const float *log_fgate, const void *value,
                          const void *key, const void *query,
                          void *hidden_final, void *out, void *states,
                          void *workspace, size_t workspace_bytes);
 int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                         int64_t chunk_size, gla_dtype dtype,
+                         int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
                          const float *log_fgate, const void *value, const void *key, const void *query,
                          const void *states, const void *dhidden_final, const void *dout,
                          void *dhidden_init, float *dlog_fgate, void *dvalue, void *dkey, void *dquery,

@@ -27,7 +27,13 @@ def test_header_symbols_are_exported_and_typed():
         assert hasattr(lib, n), f"{n} declared in gla_hip.h but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature in gla_jax_amd/_lib.py"
     assert sorted(_lib.SIGNATURES) == names
-    assert _lib.load().gla_abi_version() == 1
+    header = open(os.path.join(ROOT, "include", "gla_hip.h")).read()
+    assert _lib.load().gla_abi_version() == _lib.ABI_VERSION == int(
+        re.search(r"#define GLA_HIP_ABI_VERSION (\d+)", header).group(1))
+    # every ctypes signature lists as many arguments as the header declares
+    from tests.test_xla_ffi_shim import declared
+    for n, count in declared().items():
+        assert len(_lib.SIGNATURES[n][1]) == count, f"{n}: {len(_lib.SIGNATURES[n][1])} ctypes arguments, {count} declared"
 
 
 def test_status_strings():
@@ -66,24 +72,26 @@ def test_entry_points_reject_bad_arguments_without_touching_the_gpu():
     a = (ctypes.addressof(buf) + 15) & ~15          # a 16-byte aligned, non-null host address (never dereferenced)
     # NULL pointers
     assert lib.gla_cumsum_f32(None, None, None, a, 1, 8, 8, 0) == -1
-    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 1, 1, 0, None, a, a, a, a, a, a) == -1
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 1, 1, 1, 0, None, a, a, a, a, a, a) == -1
     # shapes / dtypes
     assert lib.gla_cumsum_f32(None, a, None, a, 0, 8, 8, 0) == -2
-    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 48, 48, 1, 1, 0, a, a, a, a, a, a, a) == -2
-    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 32, 1, 1, 0, a, a, a, a, a, a, a) == -2   # DK != DV
-    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 5, 1, 0, a, a, a, a, a, a, a) == -3
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 48, 48, 1, 1, 1, 0, a, a, a, a, a, a, a) == -2
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 32, 1, 1, 1, 0, a, a, a, a, a, a, a) == -2   # DK != DV
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 5, 1, 1, 0, a, a, a, a, a, a, a) == -3
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 1, 7, 1, 0, a, a, a, a, a, a, a) == -3   # hidden dtype
     assert lib.gla_rnn_scan_f32(None, a, a, None, None, None, a, 1, 4, 4, 0, 0) == -2
     assert lib.gla_rnn_scan_f32(None, a, a + 4, None, None, None, a, 1, 4, 4, 8, 0) == -6      # 16-byte rows
     # misaligned
-    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 1, 1, 0, a + 2, a, a, a, a, a, a) == -6
+    assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 1, 1, 1, 0, a + 2, a, a, a, a, a, a) == -6
     # chunk: not a power of two / not dividing T / unsupported head dim / missing workspace
-    args = lambda T, D, C: (None, 1, T, 1, D, D, C, 1, a, a, a, a, a, a, a, a)
+    args = lambda T, D, C, hd=0: (None, 1, T, 1, D, D, C, 1, hd, a, a, a, a, a, a, a, a)
     assert lib.gla_chunk_fwd(*args(256, 64, 48), a, 1 << 30) == -4
     assert lib.gla_chunk_fwd(*args(200, 64, 64), a, 1 << 30) == -4
     assert lib.gla_chunk_fwd(*args(256, 96, 64), a, 1 << 30) == -7
     assert lib.gla_chunk_fwd(*args(256, 64, 64), None, 0) == -5
     assert lib.gla_chunk_fwd(*args(256, 64, 64), a, 16) == -5
-    assert lib.gla_chunk_bwd(None, 1, 256, 1, 64, 64, 64, 1, a, a, a, a, None, a, a, a, a, a, a, a, a, 1 << 30) == -1
+    assert lib.gla_chunk_fwd(*args(256, 64, 64, hd=3), a, 1 << 30) == -3
+    assert lib.gla_chunk_bwd(None, 1, 256, 1, 64, 64, 64, 1, 1, a, a, a, a, None, a, a, a, a, a, a, a, a, 1 << 30) == -1
 
 
 def test_front_end_has_no_cpu_path():

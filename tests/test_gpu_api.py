@@ -1,11 +1,13 @@
 """Dtype and differentiation rules of the public entry points that the parity files do not exercise:
-hidden_init in a dtype of its own (hidden_final comes back in that dtype, gla.py:46, 727; the state enters the
-chunk kernels in the value dtype, gla.py:720) and the refusal of second-order gradients (the reference defines
+hidden_init in a dtype of its own (it enters the fp32 state uncast and hidden_final comes back in that dtype,
+gla.py:44-46, 89-97, 711-716, 727) and the refusal of second-order gradients (the reference defines
 first-order custom_vjp rules only, gla.py:441, 655)."""
+import numpy as np
 import pytest
 import torch
 
-from tests.util import cotangents, gpu_inputs, loss_of
+from oracle import gla_oracle as O
+from tests.util import assert_plain, cotangents, err_over_rms, gpu_inputs, loss_of, to_dev, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -16,28 +18,62 @@ def _bind(name):
             "recurrent_gla_naive": lambda *a: recurrent_gla_naive(*a, False)}[name]
 
 
-@pytest.mark.parametrize("name", ["chunk_gla", "recurrent_gla", "recurrent_gla_naive"])
-def test_fp32_hidden_init_with_bf16_arrays(name):
-    """hidden_init float32 (values that bf16 holds exactly) beside bf16 value/key/query: hidden_final and the
-    gradient of hidden_init are float32 and equal, bit for bit, what the all-bf16 call returns; `out` and the
-    other gradients do not change at all."""
+@pytest.mark.parametrize("name", ["recurrent_gla", "recurrent_gla_naive"])
+@pytest.mark.parametrize("D", [64, 32])
+def test_fp32_state_beside_bf16_arrays_is_not_rounded(name, D):
+    """A float32 hidden_init whose values bf16 does NOT hold, beside bf16 value/key/query: the recurrent paths
+    load it into their fp32 state as it is and store hidden_final in float32 (gla.py:44-46, 89-97), so the
+    final state and the gradient of the initial one match the fp64 oracle to float32 accuracy (1e-4 RMS), far
+    below the 2^-9 a cast of the state to bf16 would leave.  D=64 runs on the matrix-core kernels, D=32 on the
+    vector kernels."""
     fn = _bind(name)
     dtype = torch.bfloat16
-    (h0, g, v, k, q), dev = gpu_inputs(2, 128, 2, 64, 3.0, seed=12, dtype=dtype)
-    dhT, dout = cotangents(h0, v, 12, dtype)
-    same = [t.clone().requires_grad_(True) for t in dev]
-    hT_s, out_s = fn(*same)
-    g_s = torch.autograd.grad(loss_of(hT_s, out_s, dhT, dout), same)
-    mixed = [dev[0].float()] + [t.clone() for t in dev[1:]]
-    mixed = [t.requires_grad_(True) for t in mixed]
-    hT_m, out_m = fn(*mixed)
-    assert hT_s.dtype == dtype and hT_m.dtype == torch.float32
-    assert out_m.dtype == out_s.dtype
-    assert torch.equal(hT_m, hT_s.float()) and torch.equal(out_m, out_s)
-    g_m = torch.autograd.grad(loss_of(hT_m, out_m, dhT, dout), mixed)
-    assert g_m[0].dtype == torch.float32 and torch.equal(g_m[0], g_s[0].float())
-    for a, b in zip(g_m[1:], g_s[1:]):
-        assert a.dtype == b.dtype and torch.equal(a, b)
+    (h0, g, v, k, q), dev = gpu_inputs(2, 200, 2, D, 4.0, seed=21, dtype=dtype)
+    rng = np.random.default_rng(99)
+    h0 = rng.standard_normal(h0.shape).astype(np.float32)          # not representable in bf16
+    dhT = rng.standard_normal(h0.shape).astype(np.float32)
+    _, dout = cotangents(h0, v, 21, dtype)
+    assert np.abs(O.bf16_round(h0) - h0).max() > 1e-3
+    args = [to_dev(h0, torch.float32)] + [t.clone() for t in dev[1:]]
+    args = [t.requires_grad_(True) for t in args]
+    hT, out = fn(*args)
+    assert hT.dtype == torch.float32
+    grads = torch.autograd.grad(loss_of(hT, out, dhT, dout), args)
+    assert grads[0].dtype == torch.float32
+    exact = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout)
+    assert_plain("hidden_final", to_np(hT), exact[5], 1e-4)
+    assert_plain("dhidden_init", to_np(grads[0]), exact[0], 1e-4)
+    # and the same call with the state cast to bf16 first is measurably worse: the test would see a cast
+    hT16, _ = fn(args[0].detach().to(dtype), *[t.detach() for t in args[1:]])
+    assert err_over_rms(to_np(hT16), exact[5]) > 1e-3
+
+
+def test_chunk_fp32_state_beside_bf16_arrays_enters_the_scan_unrounded():
+    """chunk_gla hands hidden_init to the chunk scan uncast (gla.py:711-716): with keys of zero the final state
+    is exactly hidden_init times the total decay, and a float32 hidden_init that bf16 does not hold must come
+    back to float32 accuracy.  Only the copy used as the first chunk's incoming state is rounded (gla.py:720)."""
+    from gla_jax_amd import chunk_gla
+    dtype = torch.bfloat16
+    (h0, g, v, k, q), dev = gpu_inputs(2, 256, 2, 64, 4.0, seed=22, dtype=dtype)
+    rng = np.random.default_rng(98)
+    h0 = rng.standard_normal(h0.shape).astype(np.float32)
+    dhT = rng.standard_normal(h0.shape).astype(np.float32)
+    args = [to_dev(h0, torch.float32), dev[1], dev[2], torch.zeros_like(dev[3]), dev[4]]
+    args = [t.clone().requires_grad_(True) for t in args]
+    hT, out = chunk_gla(*args, 64)
+    assert hT.dtype == torch.float32 and out.dtype == dtype
+    decay = np.exp(g.astype(np.float64).sum(axis=1))                      # [B,H,DK]
+    assert_plain("hidden_final", to_np(hT), h0 * decay[..., None], 1e-5)
+    # d(hidden_init) = total decay * d(hidden_final) + (what `out` contributes: none with a zero cotangent)
+    (dh0,) = torch.autograd.grad((hT * to_dev(dhT, torch.float32)).sum(), args[:1])
+    assert dh0.dtype == torch.float32
+    assert_plain("dhidden_init", to_np(dh0), dhT * decay[..., None], 1e-5)
+    # general keys: the bf16 bound against the oracle, float32 state in and out
+    args = [to_dev(h0, torch.float32)] + [t.clone() for t in dev[1:]]
+    hT, out = chunk_gla(*args, 64)
+    eh, eo = O.recurrent_gla_naive(h0, g, v, k, q)
+    assert_plain("hidden_final", to_np(hT), eh, 2e-2)
+    assert_plain("out", to_np(out), eo, 3e-2)
 
 
 @pytest.mark.parametrize("name", ["chunk_gla", "recurrent_gla"])

@@ -35,9 +35,9 @@ def test_chunk_step_replays_from_a_graph():
 
     def step(stream, o):
         hT, out, dh0, dg, dv, dk, dq = o
-        _lib.check("gla_chunk_fwd", lib.gla_chunk_fwd(stream, B, T, H, D, D, chunk, dt, p(h0), p(g), p(v), p(k),
+        _lib.check("gla_chunk_fwd", lib.gla_chunk_fwd(stream, B, T, H, D, D, chunk, dt, dt, p(h0), p(g), p(v), p(k),
                                                       p(q), p(hT), p(out), p(states), p(ws_f), ws_f.numel()))
-        _lib.check("gla_chunk_bwd", lib.gla_chunk_bwd(stream, B, T, H, D, D, chunk, dt, p(g), p(v), p(k), p(q),
+        _lib.check("gla_chunk_bwd", lib.gla_chunk_bwd(stream, B, T, H, D, D, chunk, dt, dt, p(g), p(v), p(k), p(q),
                                                       p(states), p(dhT), p(dout), p(dh0), p(dg), p(dv), p(dk),
                                                       p(dq), p(ws_b), ws_b.numel()))
 
@@ -76,9 +76,9 @@ def test_recurrent_step_replays_from_a_graph(D):
 
     def step(stream, o):
         hT, out, dh0, dg, dv, dk, dq = o
-        _lib.check("gla_recurrent_fwd", lib.gla_recurrent_fwd(stream, B, T, H, D, D, dt, dt, 0, p(h0), p(g), p(v),
+        _lib.check("gla_recurrent_fwd", lib.gla_recurrent_fwd(stream, B, T, H, D, D, dt, dt, dt, 0, p(h0), p(g), p(v),
                                                               p(k), p(q), p(hT), p(out)))
-        _lib.check("gla_recurrent_bwd", lib.gla_recurrent_bwd(stream, B, T, H, D, D, dt, dt, 0, p(h0), p(g), p(v),
+        _lib.check("gla_recurrent_bwd", lib.gla_recurrent_bwd(stream, B, T, H, D, D, dt, dt, dt, 0, p(h0), p(g), p(v),
                                                               p(k), p(q), p(hT), p(dhT), p(dout), p(dh0), p(dg),
                                                               p(dv), p(dk), p(dq)))
 

@@ -73,10 +73,14 @@ def test_recurrent_matrix_core_path_over_gate_regimes(T, reverse, D):
     print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads)))
 
 
-def test_recurrent_gla_naive_returns_fp32_out():
+@pytest.mark.parametrize("T,D", [(50, 64), (300, 64), (150, 128), (40, 32)])
+def test_recurrent_gla_naive_returns_fp32_out(T, D):
+    """The naive flavour (gla.py:26-47): fp32 `out` (promotion at gla.py:37) to fp32 accuracy although the inputs
+    are bf16, and an fp32 cotangent for it in the backward.  D=64 and 128 run on the matrix-core kernels (the
+    fp32 accumulators stored unrounded; sequences longer than one block of steps), D=32 on the vector kernels."""
     from gla_jax_amd import recurrent_gla_naive
     dtype = torch.bfloat16
-    (h0, g, v, k, q), dev = gpu_inputs(2, 50, 2, 64, 5.0, seed=9, dtype=dtype)
+    (h0, g, v, k, q), dev = gpu_inputs(2, T, 2, D, 5.0, seed=9, dtype=dtype)
     dhT, dout = cotangents(h0, v, 2, torch.float32)
     dhT = O.bf16_round(dhT)
     hT, out, grads = run_fwd_bwd(recurrent_gla_naive, dev, to_dev(dhT, dtype), to_dev(dout, torch.float32),

@@ -101,3 +101,54 @@ def test_module_refuses_to_import_without_jax():
         importlib.import_module("gla_jax_amd.xla_ffi.gla_jax")
     from gla_jax_amd import build
     assert build.jaxlib_include() is None and build.build_xla_ffi(verbose=False) is None
+
+
+# The reference's public signatures (gla.py:657-669, 405-416, 26; ops.py:234-240, 396-403): name -> list of
+# (parameter, default or REQUIRED), in order.
+REQUIRED = object()
+REFERENCE_SIGNATURES = {
+    "chunk_gla": [("hidden_init", REQUIRED), ("log_fgate", REQUIRED), ("value", REQUIRED), ("key", REQUIRED),
+                  ("query", REQUIRED), ("chunk_size", REQUIRED), ("block_size_t", 64), ("block_size_d", 64),
+                  ("interpret", False), ("num_warps", 4), ("num_stages", 2)],
+    "recurrent_gla": [("hidden_init", REQUIRED), ("log_fgate", REQUIRED), ("value", REQUIRED), ("key", REQUIRED),
+                      ("query", REQUIRED), ("reverse", False), ("max_block_size", 64), ("num_warps", 1),
+                      ("num_stages", 1), ("interpret", False)],
+    "recurrent_gla_naive": [("hidden", REQUIRED), ("log_fgate", REQUIRED), ("value", REQUIRED), ("key", REQUIRED),
+                            ("query", REQUIRED), ("reverse", REQUIRED)],
+    "cumsum_recursive": [("src", REQUIRED), ("axis", REQUIRED), ("init", None), ("reverse", False),
+                         ("block_size_t", 2048)],
+    "rnn_recursive": [("log_fgate", REQUIRED), ("kv", REQUIRED), ("init_log_fgate", None), ("init_kv", None),
+                      ("block_size_t", 256), ("reverse", False)],
+}
+
+
+def _parsed_signatures(path):
+    """name -> [(parameter, default or REQUIRED)] of every top-level public function, from the source text."""
+    out = {}
+    for node in ast.parse(open(path).read()).body:
+        if isinstance(node, ast.FunctionDef) and not node.name.startswith("_"):
+            a = node.args
+            assert not a.posonlyargs and not a.kwonlyargs and a.vararg is None and a.kwarg is None
+            names = [x.arg for x in a.args]
+            defaults = [REQUIRED] * (len(names) - len(a.defaults)) + [ast.literal_eval(d) for d in a.defaults]
+            out[node.name] = list(zip(names, defaults))
+    return out
+
+
+def test_public_signatures_are_the_reference_ones_in_both_front_ends():
+    """Every public function of the JAX module (parsed, it cannot be imported here) and of the torch front-end
+    (inspect.signature) takes the reference's parameters, in the reference's order, with the reference's
+    defaults: a positional call written for the reference means the same thing in both."""
+    import inspect
+
+    from gla_jax_amd import gla, ops
+    jax_side = _parsed_signatures(PY)
+    for name, want in REFERENCE_SIGNATURES.items():
+        assert jax_side.get(name) == want, f"xla_ffi/gla_jax.py::{name}: {jax_side.get(name)}"
+        fn = getattr(gla, name, None) or getattr(ops, name)
+        got = [(p.name, REQUIRED if p.default is inspect.Parameter.empty else p.default)
+               for p in inspect.signature(fn).parameters.values()]
+        assert got == want, f"torch front-end {name}: {got}"
+    # nothing public in the JAX module beyond those and the two custom_vjp functions of the reference
+    assert set(jax_side) - set(REFERENCE_SIGNATURES) <= {"chunk_gla_forward_backward",
+                                                         "recurrent_gla_forward_backward"}

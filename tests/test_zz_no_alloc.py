@@ -25,10 +25,10 @@ def _run_pair(lib, _lib, B, T, H, D, chunk, seed, dtype=torch.bfloat16):
         hT, out = torch.full_like(h0, float("nan")), torch.full_like(v, float("nan"))
         states = torch.zeros(stb, dtype=torch.uint8, device="cuda")
         if static:
-            rc = lib.gla_chunk_fwd_static(st, B, T, H, D, D, chunk, dt, p(h0), p(g), p(v), p(k), p(q), p(hT), p(out),
+            rc = lib.gla_chunk_fwd_static(st, B, T, H, D, D, chunk, dt, dt, p(h0), p(g), p(v), p(k), p(q), p(hT), p(out),
                                           p(states))
         else:
-            rc = lib.gla_chunk_fwd(st, B, T, H, D, D, chunk, dt, p(h0), p(g), p(v), p(k), p(q), p(hT), p(out),
+            rc = lib.gla_chunk_fwd(st, B, T, H, D, D, chunk, dt, dt, p(h0), p(g), p(v), p(k), p(q), p(hT), p(out),
                                    p(states), p(ws), wsb)
         _lib.check("gla_chunk_fwd_static" if static else "gla_chunk_fwd", rc)
         outs.append((hT, out, states))
@@ -54,7 +54,58 @@ def test_static_entry_point_rejects_what_does_not_fit():
     assert lib.gla_chunk_fwd_workspace_bytes(B, T, H, D, D, 128, _lib.GLA_BF16) > _lib.GLA_CHUNK_FWD_STATIC_BYTES
     x = torch.zeros(16, device="cuda")                             # never touched: the call is refused on the host
     rc = lib.gla_chunk_fwd_static(torch.cuda.current_stream().cuda_stream, B, T, H, D, D, 128, _lib.GLA_BF16,
+                                  _lib.GLA_BF16,
                                   *([x.data_ptr()] * 8))
     assert rc == -5
     with pytest.raises(_lib.GlaError, match="workspace"):
         _lib.check("gla_chunk_fwd_static", rc)
+
+
+def test_static_entry_point_allocates_nothing_and_replays_from_a_graph():
+    """After a first call on the device (which looks up the array's address), a call of gla_chunk_fwd_static
+    leaves the free device memory and torch's allocator untouched, and it can be recorded into a HIP graph:
+    every replay, on new inputs copied into the same buffers and with eager work in between, equals
+    gla_chunk_fwd on those inputs bit for bit."""
+    from gla_jax_amd import _lib
+    lib = _lib.load()
+    B, T, H, D, chunk = 2, 512, 2, 128, 128
+    dt = _lib.GLA_BF16
+    p = lambda t: t.data_ptr()
+    _, dev = gpu_inputs(B, T, H, D, 2.0, seed=31, dtype=torch.bfloat16)
+    h0, g, v, k, q = dev
+    hT, out = torch.empty_like(h0), torch.empty_like(v)
+    wsb = lib.gla_chunk_fwd_workspace_bytes(B, T, H, D, D, chunk, dt)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    hT_e, out_e = torch.empty_like(h0), torch.empty_like(v)
+
+    def static(stream):
+        _lib.check("gla_chunk_fwd_static", lib.gla_chunk_fwd_static(stream, B, T, H, D, D, chunk, dt, dt, p(h0), p(g),
+                                                                    p(v), p(k), p(q), p(hT), p(out), None))
+
+    def eager():
+        _lib.check("gla_chunk_fwd", lib.gla_chunk_fwd(torch.cuda.current_stream().cuda_stream, B, T, H, D, D, chunk,
+                                                      dt, dt, p(h0), p(g), p(v), p(k), p(q), p(hT_e), p(out_e), None,
+                                                      p(ws), wsb))
+
+    static(torch.cuda.current_stream().cuda_stream)           # warm-up outside any capture
+    torch.cuda.synchronize()
+    free0, alloc0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    static(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "the call changed the free device memory"
+    assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static(torch.cuda.current_stream().cuda_stream)
+    for it in range(3):
+        _, fresh = gpu_inputs(B, T, H, D, 2.0, seed=40 + it, dtype=torch.bfloat16)
+        for dst, src in zip(dev, fresh):
+            dst.copy_(src)                                    # eager work between the replays
+        hT.fill_(float("nan"))
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        eager()
+        torch.cuda.synchronize()
+        assert torch.equal(hT, hT_e) and torch.equal(out, out_e), f"replay {it} differs from gla_chunk_fwd"
