@@ -28,7 +28,7 @@
 // state operands of a slice (32 rows of S_n [dk][dv], dS' [dk][dv] and dS' [dv][dk]) are staged in
 // the LDS tile that held the values, fetched one slice ahead; the per-row inputs of a slice (gates, q, k)
 // are fetched one slice ahead as well.
-#include "gla_chunk_common.hpp"
+#include "gla_subblock.hpp"
 #include "gla_chunk_kernels.hpp"
 
 namespace gla {
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     // ---- score blocks of both roles, cached as MFMA operands (2 registers each) -----------------------
     //   row owner:    dA^T of the earlier sub-blocks, dAx[J][j][i] = v_j . dO_i               (J < w)
     //   column owner: A_IJ (key side walked up by r_I) and dA_IJ = dAx[I] of the later ones   (I > w)
-    T4 dAx[NB], Ac[NB];
+    T4 dAx[NB], Ac[NB], Acl;
     D8 Kt[KS];                           // k e^{L_end - L_j}: B operand of the dS' product of dv
     {
 #pragma unroll
@@ -341,7 +341,9 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 dAx[I] = pack4<T>(da);
             }
         }
-        Ac[0] = pack4<T>(Aown);
+        // the own sub-block's scores enter dv = A^T dO as head + remainder: they are the largest of a column, and
+        // under strong decay they carry most of dv
+        split4<T>(Aown, Ac[0], Acl);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) Kt[ks] = pack8<T>(kch + 8 * ks);
     }
@@ -580,8 +582,13 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 if (I >= w) {
                     const T4 b4 = I == w ? Ac[0] : Ac[I];
 #pragma unroll
-                    for (int tt = 0; tt < 2; ++tt)
-                        acc[tt] = mma_t(lds_tr4(tO + L.k4 + fo + 4 * tt + 16 * I * LS, LS), b4, acc[tt]);
+                    for (int tt = 0; tt < 2; ++tt) {
+                        const T4 oa = lds_tr4(tO + L.k4 + fo + 4 * tt + 16 * I * LS, LS);
+                        if constexpr (sizeof(T) == 2) {
+                            if (I == w) acc[tt] = mma_t(oa, Acl, acc[tt]);
+                        }
+                        acc[tt] = mma_t(oa, b4, acc[tt]);
+                    }
                 }
             }
             float o[8];

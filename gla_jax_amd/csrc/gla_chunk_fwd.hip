@@ -129,7 +129,10 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
         sc[J] = pack4<T>(a);
     }
     sc[NB - 1] = pack4<T>(f32x4{0.f, 0.f, 0.f, 0.f});
-    const T4 scD = pack4<T>(accD);
+    // The own sub-block's scores enter the product with V as head + remainder: next to the diagonal the gated
+    // scores are the largest of a row, and under strong decay they carry most of the output.
+    T4 scD, scDl;
+    split4<T>(accD, scD, scDl);
     D8 qb[KS];                           // q * exp(L_i): operand of the state term
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qb[ks] = pack8<T>(qh + 8 * ks);
@@ -150,8 +153,13 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
             if (J <= w) {
                 const T4 b4 = J == w ? scD : sc[J];
 #pragma unroll
-                for (int tt = 0; tt < 2; ++tt)
-                    acc[tt] = mma_t(lds_tr4(Vn + L.k4 + fo + 4 * tt + 16 * J * LS, LS), b4, acc[tt]);
+                for (int tt = 0; tt < 2; ++tt) {
+                    const T4 va = lds_tr4(Vn + L.k4 + fo + 4 * tt + 16 * J * LS, LS);
+                    if constexpr (sizeof(T) == 2) {
+                        if (J == w) acc[tt] = mma_t(va, scDl, acc[tt]);
+                    }
+                    acc[tt] = mma_t(va, b4, acc[tt]);
+                }
             }
         }
         float o[8];

@@ -16,10 +16,12 @@ gla.py:782, which the gradient kernel formed as sum_v dS' * S_{n+1} from the STO
 carries the bf16 rounding of a whole state, where the reference's two terms carry the rounding of a decayed
 state and of single key rows.  The kernel now forms the two terms as the reference does (gla_chunk_bwd.hip).
 
-What stays open is listed apart and expected to fail: one case of a further 300 whose dvalue sits at 1.505 x the
-emulated reference's error (bound 1.5 x, 0.3 % over).  dvalue's error is the bf16 rounding of the score blocks,
-which the reference rounds the same way (gla.py:1029); the two maxima are independent samples and their ratio
-scatters around 1."""
+A last one (of a further 300) had dvalue at 1.505 x the emulated reference's error (bound 1.5 x): the bf16
+rounding of the score blocks as the operand of dv = A^T dO, under strong decay, where the own sub-block's scores
+carry most of dv.  Those now enter that product (and out = A V in the forward) as bf16 head + remainder.
+
+OPEN_CASES lists cases that are known to fail and not fixed; they are expected failures (strict: a case that
+starts to pass must be moved to SWEEP_CASES).  It is empty."""
 import numpy as np
 import pytest
 import torch
@@ -61,19 +63,18 @@ SWEEP_CASES = {
     # third family: the chunk-level term of d(log_fgate)
     "s505_c115": (3, 384, 2, 128, 128, 5.0, 506015, 115, None, 0.0, "dlog_fgate"),
     "s606_c64": (1, 64, 1, 64, 32, -2.0, 606964, 64, None, 0.0, "dlog_fgate"),
-}
-
-
-# found by a sweep, out of bounds, not fixed (see the module docstring)
-OPEN_CASES = {
+    # dvalue under strong decay: the own sub-block's scores as the operand of dv = A^T dO
     "s707_c228": (2, 256, 1, 64, 128, 1.0, 708128, 228, None, 0.0, "dvalue"),
 }
 
 
+# found by a sweep, out of bounds, not fixed (see the module docstring)
+OPEN_CASES = {}
+
+
 @pytest.mark.parametrize("case", sorted(SWEEP_CASES) + [
-    pytest.param(c, marks=pytest.mark.xfail(reason="dvalue 1.505 x the emulated reference (bound 1.5 x): the bf16 "
-                                                   "rounding of the score blocks, shared with the reference",
-                                            strict=False)) for c in sorted(OPEN_CASES)])
+    pytest.param(c, marks=pytest.mark.xfail(reason="known to be out of bounds, see the module docstring",
+                                            strict=True)) for c in sorted(OPEN_CASES)])
 def test_chunk_sweep_case(case):
     from gla_jax_amd import chunk_gla
     B, T, H, D, chunk, shift, seed, cseed, rows, val, _ = {**SWEEP_CASES, **OPEN_CASES}[case]
