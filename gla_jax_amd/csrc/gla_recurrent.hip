@@ -425,8 +425,8 @@ static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, i
                       const void *dout, void *dh0, float *dg, void *dv, void *dk, void *dq)
 {
     dim3 grid(H, B), block(DK / 16 * 64);
-    // bf16 data at head dimensions 64 and 128 runs both sweeps on the matrix cores
-    if (sizeof(T) == 2 && sizeof(TO) == 2 && (DK == 64 || DK == 128)) {
+    // bf16 data at head dimensions 64 and 128 runs both sweeps on the matrix cores, whatever the type of dout
+    if (sizeof(T) == 2 && (DK == 64 || DK == 128)) {
         const int dout_f32 = sizeof(TO) == 4;
         int e = launch_recurrent_stream_dq(st, B, T_len, H, DK, reverse, hdt, dout_f32, h0, g, v, k, q, dhT, dout, dq,
                                            dg);

@@ -45,6 +45,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
     T *Sl = Sh + D * LS;                           // [D][LS]  ... and remainder
     T *xs = Sl + D * LS;                           // [NB][2][16][XS] per-wave scratch (hard gates only)
     float *rtab = reinterpret_cast<float *>(xs + NB * 2 * 16 * XS);   // [NB][D] exp(tau_m)
+    constexpr bool kSplitDout = sizeof(TO) == 4;   // an fp32 dout enters the products as bf16 head + remainder
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
         const bool valid = validN;
         const int64_t row = rowN;
         float p[NV], dqo[NV];                // l_i; the own sub-block's part of dq (already scaled)
-        D8 qf[KS], kf[KS], dof[KS];
+        D8 qf[KS], kf[KS], dof[KS], dofl[KS];   // dofl: what the bf16 rounding of an fp32 dout row leaves over
         T4 lowTh, lowTl;                     // dA^T of the own sub-block below the diagonal (one anchor)
         bool one_anchor;
         {
@@ -132,6 +133,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
                 kf[ks] = kN[ks];
                 vf[ks] = vN[ks];
                 dof[ks] = dN[ks].operand();
+                if constexpr (kSplitDout) dofl[ks] = dN[ks].remainder();
                 st8(Vn + wrow + 32 * ks, vf[ks]);
             }
 
@@ -139,6 +141,10 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
             f32x4 dAn = {0.f, 0.f, 0.f, 0.f}, dAt = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
+                if constexpr (kSplitDout) {
+                    dAn = mma_d(dofl[ks], vf[ks], dAn);
+                    dAt = mma_d(vf[ks], dofl[ks], dAt);
+                }
                 dAn = mma_d(dof[ks], vf[ks], dAn);
                 dAt = mma_d(vf[ks], dof[ks], dAt);
             }
@@ -224,7 +230,11 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
             f32x4 da = {0.f, 0.f, 0.f, 0.f};
             if (J < w) {
 #pragma unroll
-                for (int k2 = 0; k2 < KS; ++k2) da = mma_d(ld8(Vn + L.nat + 16 * J * LS + 32 * k2), dof[k2], da);
+                for (int k2 = 0; k2 < KS; ++k2) {
+                    const D8 vj = ld8(Vn + L.nat + 16 * J * LS + 32 * k2);
+                    if constexpr (kSplitDout) da = mma_d(vj, dofl[k2], da);
+                    da = mma_d(vj, dof[k2], da);
+                }
             }
             split4<T>(da, dah[J], dal[J]);
         }
@@ -240,7 +250,9 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt) {
                     acc[tt] = mma_d(ld8(Sl + L.own + (fo + 4 * tt) * LS + 32 * k2), dof[k2], acc[tt]);
-                    acc[tt] = mma_d(ld8(Sh + L.own + (fo + 4 * tt) * LS + 32 * k2), dof[k2], acc[tt]);
+                    const D8 sh = ld8(Sh + L.own + (fo + 4 * tt) * LS + 32 * k2);
+                    if constexpr (kSplitDout) acc[tt] = mma_d(sh, dofl[k2], acc[tt]);
+                    acc[tt] = mma_d(sh, dof[k2], acc[tt]);
                 }
             }
 #pragma unroll
@@ -368,6 +380,8 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
     float *rtab = reinterpret_cast<float *>(xs + NB * 2 * 16 * XS);   // [NB][D] exp(tau_m)
     float *dltab = rtab + NB * D;                  // [NB][D] sub-block sums of q*dq - k*dk
     float *runtab = dltab + NB * D;                // [2][D]  sum over the later blocks of q*dq - k*dk, double-buffered
+    constexpr bool kSplitDout = sizeof(TO) == 4;   // an fp32 dout enters the products as bf16 head + remainder
+    T *tOl = reinterpret_cast<T *>(runtab + 2 * D);   // [C][LS]  the remainder of dout (fp32 dout only)
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -463,6 +477,12 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                 vf[ks] = vN[ks];
                 dof[ks] = dN[ks].operand();
                 st8(tO + wrow + 32 * ks, dof[ks]);
+                if constexpr (kSplitDout) {
+                    const D8 dofl = dN[ks].remainder();
+                    st8(tOl + wrow + 32 * ks, dofl);
+                    dAn = mma_d(dofl, vf[ks], dAn);
+                    dAt = mma_d(vf[ks], dofl, dAt);
+                }
             }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -616,6 +636,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                         split8<T>(kch + 8 * ks, kh, kl);
                         a = mma_d_split(ld8(Qh + L.nat + 16 * I * LS + 32 * ks), ld8(Ql + L.nat + 16 * I * LS + 32 * ks),
                                         kh, kl, a);
+                        if constexpr (kSplitDout) da = mma_d(ld8(tOl + L.nat + 16 * I * LS + 32 * ks), vf[ks], da);
                         da = mma_d(ld8(tO + L.nat + 16 * I * LS + 32 * ks), vf[ks], da);
                         f32x8 rr = ld8(rtab + I * D + 32 * ks + 8 * c);
 #pragma unroll
@@ -651,6 +672,8 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                         for (int tt = 0; tt < 2; ++tt) {
                             const T4 oa = lds_tr4(tO + L.k4 + fo + 4 * tt + 16 * I * LS, LS);
                             acc[tt] = mma_t(oa, bl4, acc[tt]);
+                            if constexpr (kSplitDout)
+                                acc[tt] = mma_t(lds_tr4(tOl + L.k4 + fo + 4 * tt + 16 * I * LS, LS), bh4, acc[tt]);
                             acc[tt] = mma_t(oa, bh4, acc[tt]);
                         }
                     }
@@ -725,6 +748,8 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                     for (int e = 0; e < 4; ++e) DS[i][nt][e] *= rr[e];
                     const T4 ob = lds_tr4(tO + ptl + 16 * I * LS + 16 * nt, LS);
                     DS[i][nt] = mma_t(qal, ob, DS[i][nt]);
+                    if constexpr (kSplitDout)
+                        DS[i][nt] = mma_t(qah, lds_tr4(tOl + ptl + 16 * I * LS + 16 * nt, LS), DS[i][nt]);
                     DS[i][nt] = mma_t(qah, ob, DS[i][nt]);
                 }
             }
@@ -786,7 +811,8 @@ static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, int 
     typedef BT T;
     constexpr int LS = TileGeom<T, D>::kStride;
     constexpr int XS = 32 + 16 / (int)sizeof(T);
-    const size_t lds = ((size_t)(3 * C + 2 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
+    const size_t lds = ((size_t)(3 * C + 2 * D + (sizeof(TO) == 4 ? C : 0)) * LS + (size_t)(C / 16) * 2 * 16 * XS) *
+                           sizeof(T) +
                        (size_t)(2 * (C / 16) + 2) * D * sizeof(float);
     auto kern = recurrent_stream_rev_kernel<TO, C, D>;
     static LdsGrant grant;

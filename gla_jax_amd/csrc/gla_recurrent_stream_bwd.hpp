@@ -11,21 +11,30 @@ typedef __bf16 BT;
 
 // Eight consecutive elements of a `dout` row on their way from memory to the bf16 tile the products read.  TO is
 // the element type of `dout`: bf16 for recurrent_gla; float for the recurrent_gla_naive flavour, whose `out` is
-// fp32 (gla.py:37) and so is its cotangent.  There the row is rounded to bf16 where it enters the tile (every
-// gradient it feeds is stored in bf16 or is a sum over many steps, so the 2^-9 of that rounding stays below the
-// storage rounding of the results).
+// fp32 (gla.py:37) and so is its cotangent.  There the row enters every product as bf16 head + remainder (a second
+// tile), like the other operands that are not bf16 numbers to begin with: with the head alone dvalue came out at
+// 1.5 x its storage rounding.
 template <typename TO> struct DoutRow;
 template <> struct DoutRow<BT> {
     bf16x8 raw;
     __device__ __forceinline__ void load(const BT *p) { raw = ld8(p); }
     __device__ __forceinline__ void zero() { const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; raw = pack8<BT>(z); }
     __device__ __forceinline__ bf16x8 operand() const { return raw; }
+    __device__ __forceinline__ bf16x8 remainder() const { return raw; }   // never used: a bf16 row has none
 };
 template <> struct DoutRow<float> {
     f32x8 raw;
     __device__ __forceinline__ void load(const float *p) { raw = ld8(p); }
     __device__ __forceinline__ void zero() { const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; raw = pack8<float>(z); }
     __device__ __forceinline__ bf16x8 operand() const { return pack8<BT>(raw.v); }
+    __device__ __forceinline__ bf16x8 remainder() const
+    {
+        float lo[8];
+        unpack8(pack8<BT>(raw.v), lo);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) lo[e] = raw.v[e] - lo[e];
+        return pack8<BT>(lo);
+    }
 };
 
 // One level (half-width H) of the dyadic recursion of a 16-token sub-block on a 32-feature slice: the mixed

@@ -44,6 +44,8 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
     T *Sl = Sh + D * LS;                           // [D][LS]  ... and remainder
     T *xs = Sl + D * LS;                           // [NW][2][16][XS] per-wave scratch (hard gates only)
     float *rtab = reinterpret_cast<float *>(xs + NW * 2 * 16 * XS);   // [NB][D] exp(tau_m)
+    constexpr bool kSplitDout = sizeof(TO) == 4;   // an fp32 dout enters the products as bf16 head + remainder
+    T *tOl = reinterpret_cast<T *>(rtab + NB * D); // [C][LS]  the remainder of dout (fp32 dout only)
 
     const int lane = threadIdx.x & 63;
     const int W = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -149,6 +151,7 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
             unpack8(kN, bq);
             st8(Vn + wrow + fo, vN);
             st8(tO + wrow + fo, dN.operand());
+            if constexpr (kSplitDout) st8(tOl + wrow + fo, dN.remainder());
 
             // gate prefix, totals through the wave's half of the table row, one anchor or not
             float *rt = rtab + I * D + fo + 8 * c;
@@ -203,12 +206,13 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
         auto chain = [&](auto Ic) {
             constexpr int I_ = decltype(Ic)::value;
             constexpr int NJ = I_ > 0 ? I_ : 1;
-            D8 dof[KS], vf[KS], vJ[NJ][KS], sLo[KS][2], sHi[KS][2];
+            D8 dof[KS], dofl[KS], vf[KS], vJ[NJ][KS], sLo[KS][2], sHi[KS][2];
             f32x8 rr[NJ];
             T4 kh[NJ][2], kl[NJ][2], kho[2], klo[2];
 #pragma unroll
             for (int k2 = 0; k2 < KS; ++k2) {
                 dof[k2] = ld8(tO + wrow + 32 * k2);
+                if constexpr (kSplitDout) dofl[k2] = ld8(tOl + wrow + 32 * k2);
                 vf[k2] = ld8(Vn + wrow + 32 * k2);
             }
 #pragma unroll
@@ -242,7 +246,10 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
             // dA^T of the pairs with the earlier sub-blocks, [j][i] = v_j . do_i.
             f32x4 dAt = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int k2 = 0; k2 < KS; ++k2) dAt = mma_d(vf[k2], dof[k2], dAt);
+            for (int k2 = 0; k2 < KS; ++k2) {
+                if constexpr (kSplitDout) dAt = mma_d(vf[k2], dofl[k2], dAt);
+                dAt = mma_d(vf[k2], dof[k2], dAt);
+            }
             // the state term of the slice
             f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
@@ -250,6 +257,7 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt) {
                     acc[tt] = mma_d(sLo[k2][tt], dof[k2], acc[tt]);
+                    if constexpr (kSplitDout) acc[tt] = mma_d(sHi[k2][tt], dofl[k2], acc[tt]);
                     acc[tt] = mma_d(sHi[k2][tt], dof[k2], acc[tt]);
                 }
             __builtin_amdgcn_sched_barrier(0);
@@ -261,7 +269,10 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
             for (int J = 0; J < I_; ++J) {
                 f32x4 da = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int k2 = 0; k2 < KS; ++k2) da = mma_d(vJ[J][k2], dof[k2], da);
+                for (int k2 = 0; k2 < KS; ++k2) {
+                    if constexpr (kSplitDout) da = mma_d(vJ[J][k2], dofl[k2], da);
+                    da = mma_d(vJ[J][k2], dof[k2], da);
+                }
                 split4<T>(da, dah[J], dal[J]);
             }
             // the earlier sub-blocks in ascending order
@@ -295,7 +306,10 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_dq2_kernel(
                 // hard gates: the dyadic levels on the slice, inputs fetched again
                 f32x4 dAn = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int k2 = 0; k2 < KS; ++k2) dAn = mma_d(dof[k2], vf[k2], dAn);
+                for (int k2 = 0; k2 < KS; ++k2) {
+                    if constexpr (kSplitDout) dAn = mma_d(dofl[k2], vf[k2], dAn);
+                    dAn = mma_d(dof[k2], vf[k2], dAn);
+                }
                 const HardSliceDq hs = hard_slice_dq<XS, false>(
                     g + row, q + row, k + row, valid ? 1.f : 0.f, dd, dAt, dAn, (LdsBT)xh, (LdsBT)xl, Lx.nat, Lx.k4,
                     (LdsF32) nullptr, (LdsBT) nullptr, (LdsBT) nullptr);
@@ -392,7 +406,8 @@ static int launch_dq2(hipStream_t st, int B, int T_len, int H, int reverse, int 
     typedef BT T;
     constexpr int LS = TileGeom<T, D>::kStride;
     constexpr int XS = 32 + 16 / (int)sizeof(T);
-    const size_t lds = ((size_t)(4 * C + 2 * D) * LS + (size_t)(C / 8) * 2 * 16 * XS) * sizeof(T) +
+    const size_t lds = ((size_t)(4 * C + 2 * D + (sizeof(TO) == 4 ? C : 0)) * LS + (size_t)(C / 8) * 2 * 16 * XS) *
+                           sizeof(T) +
                        (size_t)(C / 16) * D * sizeof(float);
     auto kern = recurrent_stream_dq2_kernel<TO, C, D>;
     static LdsGrant grant;
@@ -437,6 +452,8 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
     float *dltab = rtab + NB * D;                  // [NB][D] sub-block sums of q*dq - k*dk
     float *runtab = dltab + NB * D;                // [2][D]  sum over the later blocks, double-buffered
     f32x4 *xch = reinterpret_cast<f32x4 *>(runtab + 2 * D);          // [NW][NB][64] score blocks of a slice
+    constexpr bool kSplitDout = sizeof(TO) == 4;   // an fp32 dout enters the products as bf16 head + remainder
+    T *tOl = reinterpret_cast<T *>(xch + NW * NB * 64);               // [C][LS]  the remainder of dout (fp32 dout only)
 
     const int lane = threadIdx.x & 63;
     const int W = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -532,6 +549,7 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
                 qdqN = pack8<float>(z);
             }
             st8(tO + wrow + fo, dN.operand());
+            if constexpr (kSplitDout) st8(tOl + wrow + fo, dN.remainder());
             st8(Vn + wrow + fo, vN);
 
             float *rt = rtab + J0 * D + fo + 8 * c;
@@ -593,6 +611,14 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
             for (int k2 = 0; k2 < KS; ++k2) {
                 dof[k2] = ld8(tO + wrow + 32 * k2);
                 vf[k2] = ld8(Vn + wrow + 32 * k2);
+            }
+            if constexpr (kSplitDout) {
+#pragma unroll
+                for (int k2 = 0; k2 < KS; ++k2) {
+                    const D8 dofl = ld8(tOl + wrow + 32 * k2);
+                    dAn = mma_d(dofl, vf[k2], dAn);
+                    dAt = mma_d(vf[k2], dofl, dAt);
+                }
             }
 #pragma unroll
             for (int k2 = 0; k2 < KS; ++k2) {
@@ -682,7 +708,10 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
                     split8<T>(kch, kh, kl);
                     as = mma_d_split(ld8(Qh + L.nat + 16 * I * LS + fo), ld8(Ql + L.nat + 16 * I * LS + fo), kh, kl, as);
 #pragma unroll
-                    for (int k2 = 0; k2 < KS; ++k2) da = mma_d(ld8(tO + L.nat + 16 * I * LS + 32 * k2), vf[k2], da);
+                    for (int k2 = 0; k2 < KS; ++k2) {
+                        if constexpr (kSplitDout) da = mma_d(ld8(tOl + L.nat + 16 * I * LS + 32 * k2), vf[k2], da);
+                        da = mma_d(ld8(tO + L.nat + 16 * I * LS + 32 * k2), vf[k2], da);
+                    }
                     f32x8 rr = ld8(rtab + I * D + fo + 8 * c);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) kch[e] *= rr.v[e];
@@ -738,6 +767,8 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
                     for (int tt = 0; tt < 2; ++tt) {
                         const T4 oa = lds_tr4(tO + L.k4 + fo + 4 * tt + 16 * I * LS, LS);
                         acc[tt] = mma_t(oa, bl4, acc[tt]);
+                        if constexpr (kSplitDout)
+                            acc[tt] = mma_t(lds_tr4(tOl + L.k4 + fo + 4 * tt + 16 * I * LS, LS), bh4, acc[tt]);
                         acc[tt] = mma_t(oa, bh4, acc[tt]);
                     }
                 }
@@ -807,6 +838,7 @@ __global__ __launch_bounds__(C * 8) void recurrent_stream_rev2_kernel(
                 for (int e = 0; e < 4; ++e) DS[j][e] *= rr[e];
                 const T4 ob = lds_tr4(tO + ptl + 16 * I * LS + 16 * (nt0 + j), LS);
                 DS[j] = mma_t(qal, ob, DS[j]);
+                if constexpr (kSplitDout) DS[j] = mma_t(qah, lds_tr4(tOl + ptl + 16 * I * LS + 16 * (nt0 + j), LS), DS[j]);
                 DS[j] = mma_t(qah, ob, DS[j]);
             }
         }
@@ -853,7 +885,7 @@ static int launch_rev2(hipStream_t st, int B, int T_len, int H, int reverse, int
     constexpr int LS = TileGeom<T, D>::kStride;
     constexpr int XS = 32 + 16 / (int)sizeof(T);
     constexpr int NB = C / 16, NW = 2 * NB;
-    const size_t lds = ((size_t)(6 * C + 2 * D) * LS + (size_t)NW * 2 * 16 * XS) * sizeof(T) +
+    const size_t lds = ((size_t)(6 * C + 2 * D + (sizeof(TO) == 4 ? C : 0)) * LS + (size_t)NW * 2 * 16 * XS) * sizeof(T) +
                        (size_t)(2 * NB + 2) * D * sizeof(float) + (size_t)NW * NB * 64 * sizeof(f32x4);
     auto kern = recurrent_stream_rev2_kernel<TO, C, D>;
     static LdsGrant grant;
