@@ -127,9 +127,10 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 unpack8(pfDn[u], y);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) part += x[e] * y[e];
+                static_assert(D / 8 >= 4, "at least a quad of threads holds one staged row");
                 part += dpp_f32<kDppQuadXor1>(part);
                 part += dpp_f32<kDppQuadXor2>(part);
-                part += dpp_f32<kDppRowHalfMirror>(part);
+                if constexpr (D / 8 >= 8) part += dpp_f32<kDppRowHalfMirror>(part);
                 if constexpr (D / 8 >= 16) part += dpp_f32<kDppRowMirror>(part);
                 if constexpr (D / 8 == 32) part += shfl_xor_f32(part, 16);   // a row spans two 16-lane groups
                 if (c8 == 0) {

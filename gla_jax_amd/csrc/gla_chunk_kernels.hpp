@@ -7,7 +7,8 @@ namespace gla {
 
 // (T, C, D) combinations that are compiled.  C = tokens per chunk handled by one workgroup
 // (C/16 waves), D = head dimension (DK == DV, gla.py:499).  At D = 256 the four tiles of the gradient kernel
-// fit a CU's LDS for 32 tokens only (bf16; fp32 tiles are twice as wide and do not fit at all).
+// fit a CU's LDS for 32 tokens only (bf16; fp32 tiles are twice as wide and do not fit at all).  D = 32 is the
+// smallest head dimension whose feature contractions fill one k-step of the 16x16x32 matrix instruction.
 #define GLA_FOR_EACH_CHUNK_CONFIG(M) \
     M(__bf16, 128, 128)              \
     M(__bf16, 64, 128)               \
@@ -15,9 +16,14 @@ namespace gla {
     M(__bf16, 128, 64)               \
     M(__bf16, 64, 64)                \
     M(__bf16, 32, 64)                \
+    M(__bf16, 128, 32)               \
+    M(__bf16, 64, 32)                \
+    M(__bf16, 32, 32)                \
     M(__bf16, 32, 256)               \
     M(float, 64, 64)                 \
     M(float, 32, 64)                 \
+    M(float, 64, 32)                 \
+    M(float, 32, 32)                 \
     M(float, 32, 128)
 
 template <typename T, int C, int D>

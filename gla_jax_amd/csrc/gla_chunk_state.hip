@@ -288,9 +288,11 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const
     template int launch_chunk_scan<T, D>(hipStream_t, int, int, int, int, const void *, const float *, \
                                          const float *, void *, void *, void *, int);
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUTER)
+GLA_INST_SCAN(__bf16, 32)
 GLA_INST_SCAN(__bf16, 64)
 GLA_INST_SCAN(__bf16, 128)
 GLA_INST_SCAN(__bf16, 256)
+GLA_INST_SCAN(float, 32)
 GLA_INST_SCAN(float, 64)
 GLA_INST_SCAN(float, 128)
 

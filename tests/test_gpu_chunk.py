@@ -32,6 +32,11 @@ CASES = [
     (torch.bfloat16, 1, 64, 1, 64, 64, 3.0),
     (torch.bfloat16, 2, 160, 2, 256, 32, 4.0),      # head dimension 256 (32-token tiles)
     (torch.bfloat16, 1, 256, 1, 256, 128, 0.0),     # the same under strong decay
+    (torch.bfloat16, 2, 256, 3, 32, 128, 3.0),      # head dimension 32: one k-step per feature contraction
+    (torch.bfloat16, 1, 192, 2, 32, 64, 0.0),       # ... 64-token tiles, strong decay
+    (torch.bfloat16, 1, 96, 1, 32, 32, 5.0),        # ... 32-token tiles
+    (torch.float32, 2, 192, 2, 32, 64, 2.0),        # ... fp32
+    (torch.float32, 1, 96, 2, 32, 32, 0.0),
 ]
 
 
