@@ -11,6 +11,7 @@ namespace gla {
 
 struct ChunkPlan {
     int C = 0;       // tokens per workgroup actually used (a divisor of chunk_size)
+    int D = 0;       // head dimension the kernels work on: DK, or 32 for DK = 16 (rows padded by zeros on the way in)
     size_t prod = 0, decay = 0, states = 0;   // byte sizes, each rounded up to 256
     size_t resid = 0;                         // the forward residual: N + 1 states per (b,h), the last one final
 };
@@ -32,15 +33,17 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
     if (DK != DV) return GLA_ERR_SHAPE;                      // gla.py:499
     if (!is_pow2(chunk) || T % chunk != 0) return GLA_ERR_CHUNK;   // gla.py:500, 674
     if (chunk < 32) return GLA_ERR_UNSUPPORTED;
-    // largest tile built: 128 tokens for bf16 (32 at D=256), for fp32 (tiles twice as wide) 64 at D=64 and 32 at D=128
+    // largest tile built: 128 tokens for bf16 (32 at D=256), for fp32 (tiles twice as wide) 64 at D<=64 and 32 at D=128
     int64_t C = dtype == GLA_BF16 ? (DK > 128 ? 32 : 128) : (DK > 64 ? 32 : 64);
     while (T % C != 0) C /= 2;                               // chunk >= 32 divides T, so this stops at 32 or above
-    bool ok = false;
-#define GLA_PLAN_CASE(T_, C_, D_) \
-    if (((dtype == GLA_BF16) == (sizeof(T_) == 2)) && C == C_ && DK == D_) ok = true;
+    int Dk = 0;
+#define GLA_PLAN_CASE(T_, C_, D_, DM_) \
+    if (((dtype == GLA_BF16) == (sizeof(T_) == 2)) && C == C_ && DK == DM_) Dk = D_;
     GLA_FOR_EACH_CHUNK_CONFIG(GLA_PLAN_CASE)
 #undef GLA_PLAN_CASE
-    if (!ok) return GLA_ERR_UNSUPPORTED;
+    if (!Dk) return GLA_ERR_UNSUPPORTED;
+    plan->D = Dk;
+    DK = DV = Dk;                                            // the library's own buffers are sized for the kernels' D
     const size_t N = (size_t)(T / C);
     if ((int64_t)N * H > 0x7fffffffLL) return GLA_ERR_SHAPE;   // chunks x heads is the grid's x extent
     const size_t esz = dtype == GLA_BF16 ? 2 : 4;
@@ -52,11 +55,12 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
     return GLA_OK;
 }
 
-template <typename F> static int dispatch(int dtype, int C, int D, F &&f)
+template <typename F> static int dispatch(int dtype, int C, int DM, F &&f)
 {
-#define GLA_DISPATCH_CASE(T_, C_, D_)                                           \
-    if (((dtype == GLA_BF16) == (sizeof(T_) == 2)) && C == C_ && D == D_)       \
-        return f(T_{}, std::integral_constant<int, C_>{}, std::integral_constant<int, D_>{});
+#define GLA_DISPATCH_CASE(T_, C_, D_, DM_)                                      \
+    if (((dtype == GLA_BF16) == (sizeof(T_) == 2)) && C == C_ && DM == DM_)     \
+        return f(T_{}, std::integral_constant<int, C_>{}, std::integral_constant<int, D_>{},            \
+                 std::integral_constant<int, DM_>{});
     GLA_FOR_EACH_CHUNK_CONFIG(GLA_DISPATCH_CASE)
 #undef GLA_DISPATCH_CASE
     return GLA_ERR_UNSUPPORTED;
@@ -140,19 +144,20 @@ extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t
     void *statesT = (void *)(ws + p.prod + p.decay);   // [dv][dk], consumed by the output kernel
     hipStream_t st = (hipStream_t)stream;
     const int N = (int)(T / p.C);
-    return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d) -> int {
+    return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d, auto dm) -> int {
         typedef decltype(t) E;
-        constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value;
+        constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value, DM_ = decltype(dm)::value;
         int e = 0;
         if (stages & 1)
-            e = launch_chunk_outer<E, C_, D_>(st, 0, (int)B, (int)T, (int)H, log_fgate, value, key, prodT, decay);
+            e = launch_chunk_outer<E, C_, D_, DM_>(st, 0, (int)B, (int)T, (int)H, log_fgate, value, key, prodT, decay);
         if (e) return e;
         if (stages & 2)
-            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 0, hidden_dtype, hidden_init, prodT, decay, statesT,
-                                         states, hidden_final, 1);
+            e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 0, hidden_dtype, hidden_init, prodT, decay, statesT,
+                                              states, hidden_final, 1);
         if (e) return e;
         if (stages & 4)
-            e = launch_chunk_out<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, statesT, out);
+            e = launch_chunk_out<E, C_, D_, DM_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, statesT,
+                                                 out);
         return e;
     });
 }
@@ -212,20 +217,20 @@ extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t
     void *dstatesN = (void *)(ws + p.prod + p.decay + p.states); // the same, [dk][dv]
     hipStream_t st = (hipStream_t)stream;
     const int N = (int)(T / p.C);
-    return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d) -> int {
+    return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d, auto dm) -> int {
         typedef decltype(t) E;
-        constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value;
+        constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value, DM_ = decltype(dm)::value;
         int e = 0;
         if (stages & 1)
-            e = launch_chunk_outer<E, C_, D_>(st, 1, (int)B, (int)T, (int)H, log_fgate, dout, query, prodT, decay);
+            e = launch_chunk_outer<E, C_, D_, DM_>(st, 1, (int)B, (int)T, (int)H, log_fgate, dout, query, prodT, decay);
         if (e) return e;
         if (stages & 2)
-            e = launch_chunk_scan<E, D_>(st, (int)(B * H), N, 1, hidden_dtype, dhidden_final, prodT, decay, dstatesT,
-                                         dstatesN, dhidden_init, 0);
+            e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 1, hidden_dtype, dhidden_final, prodT, decay,
+                                              dstatesT, dstatesN, dhidden_init, 0);
         if (e) return e;
         if (stages & 4)
-            e = launch_chunk_grad<E, C_, D_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,
-                                             states, dstatesT, dstatesN, dlog_fgate, dvalue, dkey, dquery);
+            e = launch_chunk_grad<E, C_, D_, DM_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,
+                                                  states, dstatesT, dstatesN, dlog_fgate, dvalue, dkey, dquery);
         return e;
     });
 }

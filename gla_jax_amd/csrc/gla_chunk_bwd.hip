@@ -33,7 +33,7 @@
 
 namespace gla {
 
-template <typename T, int C, int D>
+template <typename T, int C, int D, int DM>
 __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k,
     const T *__restrict__ q, const T *__restrict__ dout, const T *__restrict__ statesN,
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const int h = blockIdx.x % H, n = blockIdx.x / H, b = blockIdx.y;
     const int N = T_len / C;
     const int64_t tok = (int64_t)b * T_len + (int64_t)n * C + 16 * w + r;
-    const int64_t rowoff = (tok * H + h) * D;
+    const int64_t rowoff = (tok * H + h) * DM;     // DM features per row in memory (DM < D: see RowMap)
     const int64_t bhn = ((int64_t)b * H + h) * N + n;
     const TrLane<T> L = make_tr_lane<T>(LS);
     const TrLane<T> Lx = make_tr_lane<T>(XS);
@@ -105,9 +105,9 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
         }
     };
     auto row_fetch = [&](int slice) {
-        gN = ld8(refetch(g + rowoff) + 32 * slice + 8 * c);
-        qN = ld8(refetch(q + rowoff) + 32 * slice + 8 * c);
-        kN = ld8(refetch(k + rowoff) + 32 * slice + 8 * c);
+        gN = ld8_row<D, DM>(refetch(g + rowoff) + 32 * slice, c);
+        qN = ld8_row<D, DM>(refetch(q + rowoff) + 32 * slice, c);
+        kN = ld8_row<D, DM>(refetch(k + rowoff) + 32 * slice, c);
     };
     auto stage_store = [&](int slice) {
 #pragma unroll
@@ -157,19 +157,19 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
         D8 qf[KS], kf[KS], dof[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            f32x8 gg = ld8(g + rowoff + 32 * ks + 8 * c);
+            f32x8 gg = ld8_row<D, DM>(g + rowoff + 32 * ks, c);
 #pragma unroll
             for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
         }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            qf[ks] = ld8(q + rowoff + 32 * ks + 8 * c);
-            kf[ks] = ld8(k + rowoff + 32 * ks + 8 * c);
+            qf[ks] = ld8_row<D, DM>(q + rowoff + 32 * ks, c);
+            kf[ks] = ld8_row<D, DM>(k + rowoff + 32 * ks, c);
         }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            vf[ks] = ld8_once(v + rowoff + 32 * ks + 8 * c);
-            dof[ks] = ld8_once(dout + rowoff + 32 * ks + 8 * c);
+            vf[ks] = ld8_row_once<D, DM>(v + rowoff + 32 * ks, c);
+            dof[ks] = ld8_row_once<D, DM>(dout + rowoff + 32 * ks, c);
         }
         stage_fetch(0);
 
@@ -245,7 +245,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             own_dA();
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                f32x8 gg = ld8(refetch(g + rowoff) + 32 * ks + 8 * c);
+                f32x8 gg = ld8_row<D, DM>(refetch(g + rowoff) + 32 * ks, c);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) { p[8 * ks + e] = gg.v[e] * kLog2e; s[8 * ks + e] = 0.f; }
             }
@@ -522,7 +522,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 o[e] = fast_exp2(p8[e]) * hacc + dq8[e];
                 dl8[e] += qr[e] * hacc;
             }
-            st8_once(dq + rowoff + fo + 8 * c, pack8<T>(o));
+            st8_row_once<D, DM>(dq + rowoff + fo, c, pack8<T>(o));
         }
         // -- dk: state term V dS'^T first, then the later sub-blocks in descending order
         {
@@ -567,7 +567,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 o[e] = fast_exp2(s8[e]) * hacc + dk8[e];
                 dl8[e] -= krt[e] * hacc;
             }
-            st8_once(dk + rowoff + fo + 8 * c, pack8<T>(o));
+            st8_row_once<D, DM>(dk + rowoff + fo, c, pack8<T>(o));
         }
         // -- dv: state term K~ dS' first, then the own and the later sub-blocks
         {
@@ -595,7 +595,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             float o[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
-            st8_once(dv + rowoff + fo + 8 * c, pack8<T>(o));
+            st8_row_once<D, DM>(dv + rowoff + fo, c, pack8<T>(o));
         }
         // -- dL of the slice is complete: reverse cumsum inside the sub-block (gla.py:616-617), then, once
         // every wave has published its sub-block total, over the whole chunk + the chunk-level term (gla.py:782)
@@ -627,7 +627,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
 #pragma unroll
                 for (int e = 0; e < 8; ++e) o.v[e] += t.v[e];
             }
-            st8_once(dg + rowoff + fo + 8 * c, o);
+            st8_row_once<D, DM>(dg + rowoff + fo, c, o);
         }
         if (ks + 1 < KS) {
             stage_store(ks + 1);
@@ -636,7 +636,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     }
 }
 
-template <typename T, int C, int D>
+template <typename T, int C, int D, int DM>
 int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
                       const void *q, const void *dout, const void *statesN, const void *dstatesT,
                       const void *dstatesN, float *dg, void *dv, void *dk, void *dq)
@@ -648,7 +648,7 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
     const size_t lds = ((size_t)(3 * C + VR) * LS + (size_t)NB * 16 * XS) * sizeof(T) +
                        ((size_t)(3 * NB + 1) * D + NB * 32) * sizeof(float) +
                        ((C - 96) * LS >= NB * 16 * 32 || sizeof(T) != 2 ? 0 : (size_t)NB * 16 * 32 * sizeof(T));
-    auto kern = chunk_grad_kernel<T, C, D>;
+    auto kern = chunk_grad_kernel<T, C, D, DM>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(T_len / C * H, B), block(C * 4);
@@ -658,10 +658,10 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
     return launch_status();
 }
 
-#define GLA_INST_GRAD(T, C, D)                                                                           \
-    template int launch_chunk_grad<T, C, D>(hipStream_t, int, int, int, const float *, const void *,     \
-                                            const void *, const void *, const void *, const void *,     \
-                                            const void *, const void *, float *, void *, void *, void *);
+#define GLA_INST_GRAD(T, C, D, DM)                                                                       \
+    template int launch_chunk_grad<T, C, D, DM>(hipStream_t, int, int, int, const float *, const void *, \
+                                                const void *, const void *, const void *, const void *, \
+                                                const void *, const void *, float *, void *, void *, void *);
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_GRAD)
 
 }  // namespace gla

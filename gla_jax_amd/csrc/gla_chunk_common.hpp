@@ -139,6 +139,40 @@ __device__ __forceinline__ void st8_once(float *p, const f32x8 &v)
     __builtin_nontemporal_store(b, reinterpret_cast<f32x4 *>(p) + 1);
 }
 
+// Head dimension 16 runs on the kernels for 32 features.  A row of the caller's arrays then has DM = 16 features
+// where the kernel works on D = 32: the lanes that would hold features 16..31 (c >= 2) read the first features
+// of their row instead (an address inside the array) and replace what they read by zeros, which is what the
+// padded features are (a zero log-gate, key, query and value leave every result of the real features alone);
+// their results are not stored.  The chunk states, the per-chunk products and the decays are the library's own
+// buffers and are kept at D x D.
+template <int D, int DM> struct RowMap {
+    static_assert(DM == D || (D == 32 && DM == 16), "padding is built for head dimension 16 only");
+    static constexpr bool kPadded = DM < D;
+    static __device__ __forceinline__ bool live(int c) { return !kPadded || 8 * c < DM; }
+    static __device__ __forceinline__ int col(int c) { return live(c) ? 8 * c : 0; }
+};
+// 8 features of a row: `row_ks` points at feature 32*ks of the lane's row, c is the lane's feature group.
+template <int D, int DM, typename P> __device__ __forceinline__ auto ld8_row(const P *row_ks, int c)
+{
+    auto x = ld8(row_ks + RowMap<D, DM>::col(c));
+    if constexpr (DM < D) {
+        if (!RowMap<D, DM>::live(c)) x = decltype(x){};
+    }
+    return x;
+}
+template <int D, int DM, typename P> __device__ __forceinline__ auto ld8_row_once(const P *row_ks, int c)
+{
+    auto x = ld8_once(row_ks + RowMap<D, DM>::col(c));
+    if constexpr (DM < D) {
+        if (!RowMap<D, DM>::live(c)) x = decltype(x){};
+    }
+    return x;
+}
+template <int D, int DM, typename P, typename V> __device__ __forceinline__ void st8_row_once(P *row_ks, int c, const V &v)
+{
+    if (RowMap<D, DM>::live(c)) st8_once(row_ks + 8 * c, v);
+}
+
 // LDS tiles are row-major [rows][D] with a 16-byte pad per row.
 template <typename T, int D> struct TileGeom {
     static constexpr int kStride = D + 16 / (int)sizeof(T);

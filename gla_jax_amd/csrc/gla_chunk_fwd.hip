@@ -22,7 +22,7 @@ namespace gla {
 // Resources: two tiles (keys of all but the last sub-block, values), 32 staged state rows and a table
 // fit twice into a CU's LDS, and the register budget is held to what lets two workgroups share a CU, so
 // that one loads while the other computes.
-template <typename T, int C, int D>
+template <typename T, int C, int D, int DM>
 __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C / 32))) void chunk_out_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k, const T *__restrict__ q,
     const T *__restrict__ states, T *__restrict__ out, int T_len, int H)
@@ -45,7 +45,7 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     const int h = blockIdx.x % H, n = blockIdx.x / H, b = blockIdx.y;
     const int N = T_len / C;
     const int64_t tok = (int64_t)b * T_len + (int64_t)n * C + 16 * w + r;
-    const int64_t rowoff = (tok * H + h) * D;
+    const int64_t rowoff = (tok * H + h) * DM;     // DM features per row in memory (DM < D: see RowMap)
     const TrLane<T> L = make_tr_lane<T>(LS);
     const int wrow = 16 * w * LS + L.nat;          // this lane's row of a [token][feature] tile
 
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
         // freshly loaded row makes the wave wait for every request it has out.
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            f32x8 gg = ld8(g + rowoff + 32 * ks + 8 * c);
+            f32x8 gg = ld8_row<D, DM>(g + rowoff + 32 * ks, c);
 #pragma unroll
             for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
         }
@@ -89,19 +89,23 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            qf[ks] = ld8(q + rowoff + 32 * ks + 8 * c);
-            kf[ks] = ld8(k + rowoff + 32 * ks + 8 * c);
+            qf[ks] = ld8_row<D, DM>(q + rowoff + 32 * ks, c);
+            kf[ks] = ld8_row<D, DM>(k + rowoff + 32 * ks, c);
         }
 
-        subblock_forward<T, D, false, true>(p, qf, kf, g + rowoff, q + rowoff, k + rowoff, true, rtab + w * D, Kh + wrow,
-                               w < NB - 1, nullptr, r, c, accD, qh);
+        // (the hard-gate path reads the rows again at row + 8c: the row pointers are shifted so that a padded lane
+        // lands on its row's first features, and `valid` zeroes what it reads there)
+        const int shift = RowMap<D, DM>::col(c) - 8 * c;
+        subblock_forward<T, D, false, true>(p, qf, kf, g + rowoff + shift, q + rowoff + shift, k + rowoff + shift,
+                                            RowMap<D, DM>::live(c), rtab + w * D, Kh + wrow, w < NB - 1, nullptr, r, c,
+                                            accD, qh);
     }
     // Values and the first state rows are requested only now: the registers above are free again, and
     // the other workgroup on the CU covers the wait.
     {
         D8 vf[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) vf[ks] = ld8(v + rowoff + 32 * ks + 8 * c);
+        for (int ks = 0; ks < KS; ++ks) vf[ks] = ld8_row<D, DM>(v + rowoff + 32 * ks, c);
         stage_fetch(0);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) st8(Vn + wrow + 32 * ks, vf[ks]);
@@ -165,7 +169,7 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
         float o[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
-        st8_once(out + rowoff + fo + 8 * c, pack8<T>(o));
+        st8_row_once<D, DM>(out + rowoff + fo, c, pack8<T>(o));
         if (ks + 1 < KS) {
             __syncthreads();             // every wave is done with the staged rows
             stage_store();
@@ -175,13 +179,13 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     }
 }
 
-template <typename T, int C, int D>
+template <typename T, int C, int D, int DM>
 int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
                      const void *q, const void *states, void *out)
 {
     constexpr int LS = TileGeom<T, D>::kStride;
     const size_t lds = (size_t)(2 * C - 16 + 32) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
-    auto kern = chunk_out_kernel<T, C, D>;
+    auto kern = chunk_out_kernel<T, C, D, DM>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(T_len / C * H, B), block(C * 4);
@@ -190,9 +194,9 @@ int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, co
     return launch_status();
 }
 
-#define GLA_INST_OUT(T, C, D)                                                                          \
-    template int launch_chunk_out<T, C, D>(hipStream_t, int, int, int, const float *, const void *,   \
-                                           const void *, const void *, const void *, void *);
+#define GLA_INST_OUT(T, C, D, DM)                                                                      \
+    template int launch_chunk_out<T, C, D, DM>(hipStream_t, int, int, int, const float *, const void *, \
+                                               const void *, const void *, const void *, void *);
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUT)
 
 }  // namespace gla

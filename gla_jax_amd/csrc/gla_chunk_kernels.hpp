@@ -8,38 +8,46 @@ namespace gla {
 // (T, C, D) combinations that are compiled.  C = tokens per chunk handled by one workgroup
 // (C/16 waves), D = head dimension (DK == DV, gla.py:499).  At D = 256 the four tiles of the gradient kernel
 // fit a CU's LDS for 32 tokens only (bf16; fp32 tiles are twice as wide and do not fit at all).  D = 32 is the
-// smallest head dimension whose feature contractions fill one k-step of the 16x16x32 matrix instruction.
+// smallest head dimension whose feature contractions fill one k-step of the 16x16x32 matrix instruction; head
+// dimension 16 (the smallest the reference's score kernel takes, gla.py:975) runs on those kernels with its
+// rows padded by zeros on the way in.
+// DM is the head dimension of the caller's arrays: D, or 16 on the kernels built for D = 32 (see RowMap).
 #define GLA_FOR_EACH_CHUNK_CONFIG(M) \
-    M(__bf16, 128, 128)              \
-    M(__bf16, 64, 128)               \
-    M(__bf16, 32, 128)               \
-    M(__bf16, 128, 64)               \
-    M(__bf16, 64, 64)                \
-    M(__bf16, 32, 64)                \
-    M(__bf16, 128, 32)               \
-    M(__bf16, 64, 32)                \
-    M(__bf16, 32, 32)                \
-    M(__bf16, 32, 256)               \
-    M(float, 64, 64)                 \
-    M(float, 32, 64)                 \
-    M(float, 64, 32)                 \
-    M(float, 32, 32)                 \
-    M(float, 32, 128)
+    M(__bf16, 128, 128, 128)         \
+    M(__bf16, 64, 128, 128)          \
+    M(__bf16, 32, 128, 128)          \
+    M(__bf16, 128, 64, 64)           \
+    M(__bf16, 64, 64, 64)            \
+    M(__bf16, 32, 64, 64)            \
+    M(__bf16, 128, 32, 32)           \
+    M(__bf16, 64, 32, 32)            \
+    M(__bf16, 32, 32, 32)            \
+    M(__bf16, 128, 32, 16)           \
+    M(__bf16, 64, 32, 16)            \
+    M(__bf16, 32, 32, 16)            \
+    M(__bf16, 32, 256, 256)          \
+    M(float, 64, 64, 64)             \
+    M(float, 32, 64, 64)             \
+    M(float, 64, 32, 32)             \
+    M(float, 32, 32, 32)             \
+    M(float, 64, 32, 16)             \
+    M(float, 32, 32, 16)             \
+    M(float, 32, 128, 128)
 
-template <typename T, int C, int D>
+template <typename T, int C, int D, int DM>
 int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const float *g, const void *x,
                        const void *y, float *prodT, float *decay);
 
-template <typename T, int D>
+template <typename T, int D, int DM>
 // hdt = gla_dtype of hin / hout (hidden_init and hidden_final, or their cotangents)
 int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const void *hin, const float *prodT,
                       const float *decay, void *statesT, void *statesN, void *hout, int tail);
 
-template <typename T, int C, int D>
+template <typename T, int C, int D, int DM>
 int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
                      const void *q, const void *states, void *out);
 
-template <typename T, int C, int D>
+template <typename T, int C, int D, int DM>
 int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
                       const void *q, const void *dout, const void *statesN, const void *dstatesT,
                       const void *dstatesN, float *dg, void *dv, void *dk, void *dq);

@@ -20,7 +20,7 @@ namespace gla {
 
 // Two tiles and a table fit twice into a CU's LDS; the register budget is held to what lets two
 // workgroups share a CU, so that one loads while the other computes.
-template <typename T, int C, int D, int MODE>
+template <typename T, int C, int D, int DM, int MODE>
 __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C / 32))) void chunk_outer_kernel(const float *__restrict__ g,
                                                             const T *__restrict__ x,
                                                             const T *__restrict__ y,
@@ -42,18 +42,17 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     const int h = blockIdx.x % H, n = blockIdx.x / H, b = blockIdx.y;
     const int N = T_len / C;
     const int64_t tok = (int64_t)b * T_len + (int64_t)n * C + 16 * w + r;
-    const int64_t rowoff = (tok * H + h) * D;
+    const int64_t rowoff = (tok * H + h) * DM;     // DM features per row in memory (DM < D: see RowMap)
 
     float p[NV];
     typename FragTypes<T>::d8 yf[KS], xf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        const int d0 = 32 * ks + 8 * c;
-        f32x8 gg = ld8(g + rowoff + d0);
+        f32x8 gg = ld8_row<D, DM>(g + rowoff + 32 * ks, c);
 #pragma unroll
         for (int e = 0; e < 8; ++e) p[8 * ks + e] = gg.v[e] * kLog2e;
-        yf[ks] = ld8(y + rowoff + d0);
-        xf[ks] = ld8(x + rowoff + d0);
+        yf[ks] = ld8_row<D, DM>(y + rowoff + 32 * ks, c);
+        xf[ks] = ld8_row<D, DM>(x + rowoff + 32 * ks, c);
     }
     // Gate sums inside the sub-block (log2 units).  The query side needs the inclusive prefix l_i, the key
     // side the sum over the LATER rows, tau - l_j: that one is scanned directly (a suffix scan, then one row
@@ -145,7 +144,9 @@ template <> struct Pair<float> { typedef f32x2 type; };
 
 // U = chunks whose inputs are in flight per thread: 4 when the grid fills the machine, 32 when few (b,h)
 // pairs leave it to the single thread to keep the memory system busy (long sequences, small batch).
-template <typename T, int D, int U>
+// DM: head dimension of hin / hout in memory (16 when D = 32 stands in for it: rows and columns past DM are zero
+// on the way in and are not stored on the way out; the per-chunk buffers are D x D).
+template <typename T, int D, int DM, int U>
 __global__ __launch_bounds__(64) void chunk_scan_kernel(const void *__restrict__ hin,
                                                          const float *__restrict__ prodT,
                                                          const float *__restrict__ decay,
@@ -171,8 +172,9 @@ __global__ __launch_bounds__(64) void chunk_scan_kernel(const void *__restrict__
         // the initial state enters the fp32 running state in its own element type (ops.py:396 takes it uncast,
         // gla.py:711-716); the chunk-start copy of it below is stored in the element type like every other
         // chunk-start state (gla.py:720)
-        float t[2];
-        load_hidden<2>(hin, hdt, (int64_t)bh * D * D + (dk0 + j) * D + dv0, t);
+        float t[2] = {0.f, 0.f};
+        if (DM == D || (dk0 + j < DM && dv0 < DM))
+            load_hidden<2>(hin, hdt, (int64_t)bh * DM * DM + (dk0 + j) * DM + dv0, t);
         X[0][j] = t[0];
         X[1][j] = t[1];
     }
@@ -241,11 +243,12 @@ __global__ __launch_bounds__(64) void chunk_scan_kernel(const void *__restrict__
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const float t[2] = {X[0][j], X[1][j]};
-        store_hidden<2>(hout, hdt, (int64_t)bh * D * D + (dk0 + j) * D + dv0, t);
+        if (DM == D || (dk0 + j < DM && dv0 < DM))
+            store_hidden<2>(hout, hdt, (int64_t)bh * DM * DM + (dk0 + j) * DM + dv0, t);
     }
 }
 
-template <typename T, int C, int D>
+template <typename T, int C, int D, int DM>
 int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const float *g, const void *x,
                        const void *y, float *prodT, float *decay)
 {
@@ -253,12 +256,12 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
     const size_t lds = (size_t)2 * C * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
     dim3 grid(T_len / C * H, B), block(C * 4);
     if (mode == 0) {
-        auto kern = chunk_outer_kernel<T, C, D, 0>;
+        auto kern = chunk_outer_kernel<T, C, D, DM, 0>;
         static LdsGrant grant;
         if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
         hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)x, (const T *)y, prodT, decay, T_len, H);
     } else {
-        auto kern = chunk_outer_kernel<T, C, D, 1>;
+        auto kern = chunk_outer_kernel<T, C, D, DM, 1>;
         static LdsGrant grant;
         if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
         hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)x, (const T *)y, prodT, decay, T_len, H);
@@ -266,34 +269,36 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
     return launch_status();
 }
 
-template <typename T, int D>
+template <typename T, int D, int DM>
 int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const void *hin, const float *prodT,
                       const float *decay, void *statesT, void *statesN, void *hout, int tail)
 {
     dim3 grid(BH, (D / 16) * (D / 16)), block(64);
     if ((int64_t)grid.y * BH >= 1024) {      // at least a wave per SIMD
-        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 4>), grid, block, 0, st, hin, prodT, decay,
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, 4>), grid, block, 0, st, hin, prodT, decay,
                            (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt);
     } else {
-        hipLaunchKernelGGL((chunk_scan_kernel<T, D, 32>), grid, block, 0, st, hin, prodT, decay,
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, 32>), grid, block, 0, st, hin, prodT, decay,
                            (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt);
     }
     return launch_status();
 }
 
-#define GLA_INST_OUTER(T, C, D)                                                                       \
-    template int launch_chunk_outer<T, C, D>(hipStream_t, int, int, int, int, const float *, const void *, \
-                                             const void *, float *, float *);
-#define GLA_INST_SCAN(T, D)                                                                           \
-    template int launch_chunk_scan<T, D>(hipStream_t, int, int, int, int, const void *, const float *, \
-                                         const float *, void *, void *, void *, int);
+#define GLA_INST_OUTER(T, C, D, DM)                                                                   \
+    template int launch_chunk_outer<T, C, D, DM>(hipStream_t, int, int, int, int, const float *, const void *, \
+                                                 const void *, float *, float *);
+#define GLA_INST_SCAN(T, D, DM)                                                                       \
+    template int launch_chunk_scan<T, D, DM>(hipStream_t, int, int, int, int, const void *, const float *, \
+                                             const float *, void *, void *, void *, int);
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUTER)
-GLA_INST_SCAN(__bf16, 32)
-GLA_INST_SCAN(__bf16, 64)
-GLA_INST_SCAN(__bf16, 128)
-GLA_INST_SCAN(__bf16, 256)
-GLA_INST_SCAN(float, 32)
-GLA_INST_SCAN(float, 64)
-GLA_INST_SCAN(float, 128)
+GLA_INST_SCAN(__bf16, 32, 16)
+GLA_INST_SCAN(__bf16, 32, 32)
+GLA_INST_SCAN(__bf16, 64, 64)
+GLA_INST_SCAN(__bf16, 128, 128)
+GLA_INST_SCAN(__bf16, 256, 256)
+GLA_INST_SCAN(float, 32, 16)
+GLA_INST_SCAN(float, 32, 32)
+GLA_INST_SCAN(float, 64, 64)
+GLA_INST_SCAN(float, 128, 128)
 
 }  // namespace gla

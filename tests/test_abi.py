@@ -63,7 +63,9 @@ def test_chunk_plan_and_sizes():
     # head dims built: 32, 64, 128, and 256 on 32-token tiles for bf16 only (fp32 tiles are twice as wide)
     assert lib.gla_chunk_states_bytes(B, T, H, 32, 32, 128, _lib.GLA_BF16) == B * H * (n_chunks + 1) * 32 * 32 * 2
     assert lib.gla_chunk_states_bytes(B, T, H, 32, 32, 128, _lib.GLA_F32) == B * H * (2 * n_chunks + 1) * 32 * 32 * 4
-    assert lib.gla_chunk_states_bytes(B, T, H, 16, 16, 128, _lib.GLA_BF16) == 0
+    # head dim 16 runs on the 32-feature kernels: the library's own buffers are sized for 32 x 32 states
+    assert lib.gla_chunk_states_bytes(B, T, H, 16, 16, 128, _lib.GLA_BF16) == B * H * (n_chunks + 1) * 32 * 32 * 2
+    assert lib.gla_chunk_states_bytes(B, T, H, 8, 8, 128, _lib.GLA_BF16) == 0
     assert lib.gla_chunk_states_bytes(B, T, H, 256, 256, 128, _lib.GLA_BF16) == B * H * (4 * n_chunks + 1) * 256 * 256 * 2
     assert lib.gla_chunk_states_bytes(B, T, H, 256, 256, 128, _lib.GLA_F32) == 0
     assert lib.gla_chunk_states_bytes(B, T, H, 512, 512, 128, _lib.GLA_BF16) == 0

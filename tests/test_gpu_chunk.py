@@ -37,6 +37,11 @@ CASES = [
     (torch.bfloat16, 1, 96, 1, 32, 32, 5.0),        # ... 32-token tiles
     (torch.float32, 2, 192, 2, 32, 64, 2.0),        # ... fp32
     (torch.float32, 1, 96, 2, 32, 32, 0.0),
+    (torch.bfloat16, 2, 256, 3, 16, 128, 3.0),      # head dimension 16: the 32-feature kernels, rows padded by zeros
+    (torch.bfloat16, 1, 192, 5, 16, 64, 0.0),
+    (torch.bfloat16, 3, 32, 1, 16, 32, 5.0),
+    (torch.float32, 2, 192, 2, 16, 64, 1.0),
+    (torch.float32, 1, 96, 3, 16, 32, 4.0),
 ]
 
 

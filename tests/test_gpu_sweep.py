@@ -28,7 +28,7 @@ def draw_case(rng, it):
     B, H = int(rng.integers(1, 4)), int(rng.integers(1, 5))
     shift = float(rng.choice([-2.0, 0.0, 1.0, 3.0, 5.0]))
     if kind == "chunk":
-        D = int(rng.choice([32, 64, 128, 128, 256])) if dtype == torch.bfloat16 else int(rng.choice([32, 64, 128]))
+        D = int(rng.choice([16, 32, 64, 128, 128, 256])) if dtype == torch.bfloat16 else int(rng.choice([16, 32, 64, 128]))
         chunk = int(rng.choice([32, 64, 128]))
         T = chunk * int(rng.integers(1, 5))
         reverse = False
