@@ -13,6 +13,7 @@ struct ChunkPlan {
     int C = 0;       // tokens per workgroup actually used (a divisor of chunk_size)
     int D = 0;       // head dimension the kernels work on: DK, or 32 for DK = 16 (rows padded by zeros on the way in)
     size_t prod = 0, decay = 0, states = 0;   // byte sizes, each rounded up to 256
+    size_t scale_off = 0;                     // where the products' exponents start inside the decay region
     size_t resid = 0;                         // the forward residual: N + 1 states per (b,h), the last one final
 };
 
@@ -48,8 +49,11 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
     if ((int64_t)N * H > 0x7fffffffLL) return GLA_ERR_SHAPE;   // chunks x heads is the grid's x extent
     const size_t esz = dtype == GLA_BF16 ? 2 : 4;
     plan->C = (int)C;
-    plan->prod = round256((size_t)B * H * N * DK * DV * sizeof(float));
-    plan->decay = round256((size_t)B * H * N * DK * sizeof(float));
+    // per-chunk products: float for float data, 16-bit mantissas for bf16 data; their exponents (one byte per 16
+    // values) sit behind the decays
+    plan->prod = round256((size_t)B * H * N * DK * DV * esz);
+    plan->scale_off = (size_t)B * H * N * DK * sizeof(float);
+    plan->decay = round256(plan->scale_off + (size_t)B * H * N * (DK * DV / 16));
     plan->states = round256((size_t)B * H * N * DK * DV * esz);
     plan->resid = round256((size_t)B * H * (N + 1) * DK * DV * esz);
     return GLA_OK;
@@ -139,8 +143,9 @@ extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t
     if (!workspace || workspace_bytes < p.prod + p.decay + p.states) return GLA_ERR_WORKSPACE;
     if (!aligned16(workspace) || (states && !aligned16(states))) return GLA_ERR_ALIGN;
     unsigned char *ws = (unsigned char *)workspace;
-    float *prodT = (float *)ws;
+    void *prodT = (void *)ws;
     float *decay = (float *)(ws + p.prod);
+    unsigned char *pexp = ws + p.prod + p.scale_off;
     void *statesT = (void *)(ws + p.prod + p.decay);   // [dv][dk], consumed by the output kernel
     hipStream_t st = (hipStream_t)stream;
     const int N = (int)(T / p.C);
@@ -149,11 +154,12 @@ extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t
         constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value, DM_ = decltype(dm)::value;
         int e = 0;
         if (stages & 1)
-            e = launch_chunk_outer<E, C_, D_, DM_>(st, 0, (int)B, (int)T, (int)H, log_fgate, value, key, prodT, decay);
+            e = launch_chunk_outer<E, C_, D_, DM_>(st, 0, (int)B, (int)T, (int)H, log_fgate, value, key, prodT, decay,
+                                                   pexp);
         if (e) return e;
         if (stages & 2)
-            e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 0, hidden_dtype, hidden_init, prodT, decay, statesT,
-                                              states, hidden_final, 1);
+            e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 0, hidden_dtype, hidden_init, prodT, decay, pexp,
+                                              statesT, states, hidden_final, 1);
         if (e) return e;
         if (stages & 4)
             e = launch_chunk_out<E, C_, D_, DM_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, statesT,
@@ -211,8 +217,9 @@ extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t
     if (!workspace || workspace_bytes < p.prod + p.decay + 2 * p.states) return GLA_ERR_WORKSPACE;
     if (!aligned16(workspace)) return GLA_ERR_ALIGN;
     unsigned char *ws = (unsigned char *)workspace;
-    float *prodT = (float *)ws;
+    void *prodT = (void *)ws;
     float *decay = (float *)(ws + p.prod);
+    unsigned char *pexp = ws + p.prod + p.scale_off;
     void *dstatesT = (void *)(ws + p.prod + p.decay);            // d(chunk-end state), [dv][dk]
     void *dstatesN = (void *)(ws + p.prod + p.decay + p.states); // the same, [dk][dv]
     hipStream_t st = (hipStream_t)stream;
@@ -222,10 +229,11 @@ extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t
         constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value, DM_ = decltype(dm)::value;
         int e = 0;
         if (stages & 1)
-            e = launch_chunk_outer<E, C_, D_, DM_>(st, 1, (int)B, (int)T, (int)H, log_fgate, dout, query, prodT, decay);
+            e = launch_chunk_outer<E, C_, D_, DM_>(st, 1, (int)B, (int)T, (int)H, log_fgate, dout, query, prodT, decay,
+                                                   pexp);
         if (e) return e;
         if (stages & 2)
-            e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 1, hidden_dtype, dhidden_final, prodT, decay,
+            e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 1, hidden_dtype, dhidden_final, prodT, decay, pexp,
                                               dstatesT, dstatesN, dhidden_init, 0);
         if (e) return e;
         if (stages & 4)

@@ -35,13 +35,15 @@ namespace gla {
     M(float, 32, 128, 128)
 
 template <typename T, int C, int D, int DM>
+// prodT: the per-chunk products in the library's own layout and type (gla_chunk_state.hip), pexp: their exponents
 int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const float *g, const void *x,
-                       const void *y, float *prodT, float *decay);
+                       const void *y, void *prodT, float *decay, unsigned char *pexp);
 
 template <typename T, int D, int DM>
 // hdt = gla_dtype of hin / hout (hidden_init and hidden_final, or their cotangents)
-int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const void *hin, const float *prodT,
-                      const float *decay, void *statesT, void *statesN, void *hout, int tail);
+int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const void *hin, const void *prodT,
+                      const float *decay, const unsigned char *pexp, void *statesT, void *statesN, void *hout,
+                      int tail);
 
 template <typename T, int C, int D, int DM>
 int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,

@@ -18,14 +18,35 @@
 
 namespace gla {
 
+// The per-chunk products go from the product kernel to the scan and nowhere else, so their layout and type are
+// the library's own.  Layout: the order of the matrix instruction's accumulators, [chunk][tile row mt][tile column
+// nt][lane][4]: a lane stores the 4 accumulator values of a 16x16 tile with ONE access, a wave one contiguous
+// kilobyte or half of it, and the scan's lane (one wave per tile) reads them back the same way.  Type: float for
+// float data; for bf16 data a block floating point of 16-bit mantissas with ONE exponent per tile and key
+// feature, i.e. per 16 values P[dv = 16 mt .. + 15][dk]: the exponent is that of the largest of the 16, so nothing
+// overflows whatever the size of the inputs, a key feature that is orders of magnitude larger than its neighbours
+// (or decays away) does not cost them precision, and every value is off by at most 2^-16 of the largest of its
+// 16 (the scan adds the products into an fp32 state, so what counts is the absolute error; plain half precision,
+// 2^-12 of each value, left hidden_final of a strongly decaying case at 1.6 x its storage rounding, bf16 products
+// cost the headline shape the plain 2e-2 bound).  Exponent 255 marks a group that holds a value that is not finite
+// (or beyond 2^124): the scan reads all 16 as NaN.  The exponents (one byte each) travel next to the decays.  Half the bytes of fp32 products, written and read
+// once per direction: 100 MB less per step at B4 T4096 H6 D128.
+template <typename T> struct Prod;
+template <> struct Prod<float> { typedef float type; };
+template <> struct Prod<__bf16> { typedef short type; };
+typedef __attribute__((ext_vector_type(4))) short i16x4;
+typedef __attribute__((ext_vector_type(2))) short i16x2;
+constexpr int kProdNotFinite = 255;      // the exponent byte of a group with a value that is not finite
+
 // Two tiles and a table fit twice into a CU's LDS; the register budget is held to what lets two
 // workgroups share a CU, so that one loads while the other computes.
 template <typename T, int C, int D, int DM, int MODE>
 __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C / 32))) void chunk_outer_kernel(const float *__restrict__ g,
                                                             const T *__restrict__ x,
                                                             const T *__restrict__ y,
-                                                            float *__restrict__ prodT,
-                                                            float *__restrict__ decay, int T_len, int H)
+                                                            typename Prod<T>::type *__restrict__ prodT,
+                                                            float *__restrict__ decay,
+                                                            unsigned char *__restrict__ pexp, int T_len, int H)
 {
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16;
     constexpr int LS = TileGeom<T, D>::kStride;
@@ -110,7 +131,7 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     }
     __syncthreads();
 
-    float *outp = prodT + (((int64_t)b * H + h) * N + n) * D * D;
+    const int64_t bhn = ((int64_t)b * H + h) * N + n;
     for (int mt = w; mt < NT; mt += NB) {
         f32x4 acc[NT];
 #pragma unroll
@@ -125,19 +146,48 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
                 acc[nt] = mma_t(a, bb, acc[nt]);
             }
         }
+        // acc[nt][e] = P^T[dv = 16 mt + 4c + e][dk = 16 nt + r]: stored in this order, one access per tile and lane
+        typename Prod<T>::type *outp = prodT + ((bhn * NT + mt) * NT) * 256 + lane * 4;
+        if constexpr (sizeof(T) == 4) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+            for (int nt = 0; nt < NT; ++nt) *reinterpret_cast<f32x4 *>(outp + nt * 256) = acc[nt];
+        } else {
+            unsigned char *expp = pexp + ((bhn * NT + mt) * NT) * 16 + r;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) outp[(16 * mt + 4 * c + e) * D + 16 * nt + r] = acc[nt][e];
+            for (int nt = 0; nt < NT; ++nt) {
+                // the largest magnitude of the key feature's 16 values (4 here, 4 in each of the lanes r + 16 c'); a NaN
+                // counts as infinite
+                float m = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float a = fabsf(acc[nt][e]);
+                    m = fmaxf(m, a == a ? a : __builtin_inff());
+                }
+                m = fmaxf(m, shfl_xor_f32(m, 16));
+                m = fmaxf(m, shfl_xor_f32(m, 32));
+                // m = f 2^(eb - 126) with f in [0.5, 1): times 2^(126 - eb) every value lies in (-1, 1), which the
+                // packed conversion maps to 16-bit mantissas (x 32767, rounded).  eb is held to a range in which that
+                // scale and its inverse are normal floats: an all-zero group takes the smallest exponent of the
+                // range, a group beyond it is marked as not finite.
+                int eb = (__float_as_int(m) >> 23) & 0xff;
+                eb = eb < 27 ? 27 : (eb > 250 ? kProdNotFinite : eb);
+                const float sc = __int_as_float((253 - (eb > 250 ? 250 : eb)) << 23);
+                const i16x2 lo = __builtin_amdgcn_cvt_pknorm_i16(acc[nt][0] * sc, acc[nt][1] * sc);
+                const i16x2 hi = __builtin_amdgcn_cvt_pknorm_i16(acc[nt][2] * sc, acc[nt][3] * sc);
+                *reinterpret_cast<i16x4 *>(outp + nt * 256) = i16x4{lo[0], lo[1], hi[0], hi[1]};
+                if (c == 0) expp[nt * 16] = (unsigned char)eb;
+            }
+        }
     }
 }
 
-// One thread = a 2x2 patch of the state, one block = one wave = a 16x16 tile (8x8 lanes), walked over the
-// chunks in registers.  The running state is written per chunk in BOTH orientations ([dv][dk] for products
-// contracting over dk, [dk][dv] for products contracting over dv); with 8x8 lanes of 2x2 patches every
-// store instruction fills whole 32-byte sectors either way.  Single-wave blocks spread a state over as many
-// CUs as possible: with four-wave blocks the headline shape left a third of the chip with half the work
-// (20 -> 18 us), and 8 sequences used 128 CUs (77 -> 60 us).
+// One block = one wave = one 16x16 tile of the state, walked over the chunks in registers; lane (r, c) holds
+// S[dk = 16 nt + r][dv = 16 mt + 4c .. + 3], which is where the product kernel's accumulators of that tile sit.  The
+// running state is written per chunk in BOTH orientations ([dv][dk] for products contracting over dk, [dk][dv] for
+// products contracting over dv): [dk][dv] takes the lane's 4 values as they are; for [dv][dk] neighbouring lanes
+// swap halves first, so that each stores two rows of two neighbouring dk.  Either way every store instruction fills
+// whole 32-byte sectors.  Single-wave blocks spread a state over as many CUs as possible: with four-wave blocks the
+// headline shape left a third of the chip with half the work (20 -> 18 us), and 8 sequences used 128 CUs (77 -> 60 us).
 template <typename T> struct Pair;
 template <> struct Pair<__bf16> { typedef bf16x2 type; };
 template <> struct Pair<float> { typedef f32x2 type; };
@@ -148,110 +198,104 @@ template <> struct Pair<float> { typedef f32x2 type; };
 // on the way in and are not stored on the way out; the per-chunk buffers are D x D).
 template <typename T, int D, int DM, int U>
 __global__ __launch_bounds__(64) void chunk_scan_kernel(const void *__restrict__ hin,
-                                                         const float *__restrict__ prodT,
+                                                         const typename Prod<T>::type *__restrict__ prodT,
                                                          const float *__restrict__ decay,
+                                                         const unsigned char *__restrict__ pexp,
                                                          T *__restrict__ statesT, T *__restrict__ statesN,
                                                          void *__restrict__ hout, int N, int reverse, int tail,
                                                          int hdt)
 {
     typedef typename Pair<T>::type P2;
-    constexpr int TPD = D / 32;
+    typedef typename FragTypes<T>::t4 T4;
+    typedef typename Prod<T>::type P;
+    constexpr int TPD = D / 32, NT = D / 16;
     // (b,h) runs along x, the 32x32 tiles along y: workgroups are dealt to the 8 XCDs in x-major order, so when
     // the number of (b,h) pairs is a multiple of 8 all tiles of one state meet in ONE L2.  A tile row is half a
     // 128-byte line of the bf16 states: the halves written by neighbouring tiles are then merged there and
     // leave as whole lines.
     const int bh = blockIdx.x;
     const int tile_v = (blockIdx.y >> 2) / TPD, tile_k = (blockIdx.y >> 2) % TPD;   // 32x32 tile, then its quarter
-    const int lane = threadIdx.x, wave = blockIdx.y & 3;
-    const int ti = lane >> 3, tj = lane & 7;
-    const int dv0 = 32 * tile_v + 16 * (wave >> 1) + 2 * ti;
-    const int dk0 = 32 * tile_k + 16 * (wave & 1) + 2 * tj;
-    float X[2][2];   // X[i][j] = S[dk0 + j][dv0 + i]
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        // the initial state enters the fp32 running state in its own element type (ops.py:396 takes it uncast,
-        // gla.py:711-716); the chunk-start copy of it below is stored in the element type like every other
-        // chunk-start state (gla.py:720)
-        float t[2] = {0.f, 0.f};
-        if (DM == D || (dk0 + j < DM && dv0 < DM))
-            load_hidden<2>(hin, hdt, (int64_t)bh * DM * DM + (dk0 + j) * DM + dv0, t);
-        X[0][j] = t[0];
-        X[1][j] = t[1];
-    }
-    const float *pp = prodT + (int64_t)bh * N * D * D + dv0 * D + dk0;
-    const float *dp = decay + (int64_t)bh * N * D + dk0;
+    const int mt = 2 * tile_v + ((blockIdx.y >> 1) & 1), nt = 2 * tile_k + (blockIdx.y & 1);
+    const int lane = threadIdx.x, r = lane & 15, c = lane >> 4;
+    const int dv0 = 16 * mt + 4 * c, dk = 16 * nt + r;
+    const bool in_mem = DM == D || (dk < DM && dv0 < DM);
+    float X[4] = {0.f, 0.f, 0.f, 0.f};   // X[e] = S[dk][dv0 + e]
+    // the initial state enters the fp32 running state in its own element type (ops.py:396 takes it uncast,
+    // gla.py:711-716); the chunk-start copy of it below is stored in the element type like every other
+    // chunk-start state (gla.py:720)
+    if (in_mem) load_hidden<4>(hin, hdt, (int64_t)bh * DM * DM + dk * DM + dv0, X);
+    const P *pp = prodT + (((int64_t)bh * N * NT + mt) * NT + nt) * 256 + lane * 4;   // + n * D * D
+    const float *dp = decay + (int64_t)bh * N * D + dk;                               // + n * D
+    const unsigned char *ep = pexp + (((int64_t)bh * N * NT + mt) * NT + nt) * 16 + r;   // + n * D * D / 16
     const int64_t sbase = (int64_t)bh * N * D * D;
     const int64_t sbaseN = (int64_t)bh * (N + tail) * D * D;   // tail: one more slot holds the state after the last chunk
+    const bool odd = (r & 1) != 0;
+    auto emit_n = [&](int64_t slot) {
+        T4 t = pack4<T>(f32x4{X[0], X[1], X[2], X[3]});
+        *reinterpret_cast<T4 *>(statesN + sbaseN + slot * D * D + dk * D + dv0) = t;
+    };
     auto emit = [&](int n) {
         if (statesT) {
+            // lanes r and r^1 swap halves: the even one ends up with rows dv0, dv0 + 1, the odd one with rows
+            // dv0 + 2, dv0 + 3, each for the two neighbouring dk of the pair
+            float Y[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) Y[e] = dpp_f32<kDppQuadXor1>(X[e]);
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 P2 t;
-                t[0] = X[i][0]; t[1] = X[i][1];
-                *reinterpret_cast<P2 *>(statesT + sbase + (int64_t)n * D * D + (dv0 + i) * D + dk0) = t;
+                t[0] = odd ? Y[2 + i] : X[i];
+                t[1] = odd ? X[2 + i] : Y[i];
+                *reinterpret_cast<P2 *>(statesT + sbase + (int64_t)n * D * D + (dv0 + (odd ? 2 : 0) + i) * D +
+                                        (dk & ~1)) = t;
             }
         }
-        if (statesN) {
+        if (statesN) emit_n(n);
+    };
+    auto load_p = [&](int n, f32x4 &pv, float &dc) {
+        if constexpr (sizeof(P) == 4) {
+            pv = *reinterpret_cast<const f32x4 *>(pp + (int64_t)n * D * D);
+        } else {
+            const i16x4 h4 = *reinterpret_cast<const i16x4 *>(pp + (int64_t)n * D * D);
+            const int eb = ep[(int64_t)n * (D * D / 16)];
+            const float sc = eb == kProdNotFinite ? __builtin_nanf("")
+                                                  : __int_as_float((eb + 1) << 23) * (1.f / 32767.f);   // 2^(eb - 126) / 32767
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                P2 t;
-                t[0] = X[0][j]; t[1] = X[1][j];
-                *reinterpret_cast<P2 *>(statesN + sbaseN + (int64_t)n * D * D + (dk0 + j) * D + dv0) = t;
-            }
+            for (int e = 0; e < 4; ++e) pv[e] = (float)h4[e] * sc;
         }
+        dc = dp[(int64_t)n * D];
     };
     int step = 0;
     for (; step + U <= N; step += U) {
-        f32x2 pv[U][2], dc[U];
+        f32x4 pv[U];
+        float dc[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) load_p(reverse ? N - 1 - (step + u) : step + u, pv[u], dc[u]);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int n = reverse ? N - 1 - (step + u) : step + u;
-            pv[u][0] = *reinterpret_cast<const f32x2 *>(pp + (int64_t)n * D * D);
-            pv[u][1] = *reinterpret_cast<const f32x2 *>(pp + (int64_t)n * D * D + D);
-            dc[u] = *reinterpret_cast<const f32x2 *>(dp + (int64_t)n * D);
-        }
+            emit(reverse ? N - 1 - (step + u) : step + u);
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int n = reverse ? N - 1 - (step + u) : step + u;
-            emit(n);
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) X[i][j] = dc[u][j] * X[i][j] + pv[u][i][j];
+            for (int e = 0; e < 4; ++e) X[e] = dc[u] * X[e] + pv[u][e];
         }
     }
     for (; step < N; ++step) {
         const int n = reverse ? N - 1 - step : step;
-        f32x2 p0 = *reinterpret_cast<const f32x2 *>(pp + (int64_t)n * D * D);
-        f32x2 p1 = *reinterpret_cast<const f32x2 *>(pp + (int64_t)n * D * D + D);
-        f32x2 dc = *reinterpret_cast<const f32x2 *>(dp + (int64_t)n * D);
+        f32x4 pv;
+        float dc;
+        load_p(n, pv, dc);
         emit(n);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            X[0][j] = dc[j] * X[0][j] + p0[j];
-            X[1][j] = dc[j] * X[1][j] + p1[j];
-        }
+        for (int e = 0; e < 4; ++e) X[e] = dc * X[e] + pv[e];
     }
-    if (tail && statesN) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            P2 t;
-            t[0] = X[0][j]; t[1] = X[1][j];
-            *reinterpret_cast<P2 *>(statesN + sbaseN + (int64_t)N * D * D + (dk0 + j) * D + dv0) = t;
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const float t[2] = {X[0][j], X[1][j]};
-        if (DM == D || (dk0 + j < DM && dv0 < DM))
-            store_hidden<2>(hout, hdt, (int64_t)bh * DM * DM + (dk0 + j) * DM + dv0, t);
-    }
+    if (tail && statesN) emit_n(N);
+    if (in_mem) store_hidden<4>(hout, hdt, (int64_t)bh * DM * DM + dk * DM + dv0, X);
 }
 
 template <typename T, int C, int D, int DM>
 int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const float *g, const void *x,
-                       const void *y, float *prodT, float *decay)
+                       const void *y, void *prodT, float *decay, unsigned char *pexp)
 {
+    typedef typename Prod<T>::type P;
     constexpr int LS = TileGeom<T, D>::kStride;
     const size_t lds = (size_t)2 * C * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
     dim3 grid(T_len / C * H, B), block(C * 4);
@@ -259,26 +303,33 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
         auto kern = chunk_outer_kernel<T, C, D, DM, 0>;
         static LdsGrant grant;
         if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
-        hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)x, (const T *)y, prodT, decay, T_len, H);
+        hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)x, (const T *)y, (P *)prodT, decay, pexp, T_len,
+                           H);
     } else {
         auto kern = chunk_outer_kernel<T, C, D, DM, 1>;
         static LdsGrant grant;
         if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
-        hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)x, (const T *)y, prodT, decay, T_len, H);
+        hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)x, (const T *)y, (P *)prodT, decay, pexp, T_len,
+                           H);
     }
     return launch_status();
 }
 
 template <typename T, int D, int DM>
-int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const void *hin, const float *prodT,
-                      const float *decay, void *statesT, void *statesN, void *hout, int tail)
+int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const void *hin, const void *prodT,
+                      const float *decay, const unsigned char *pexp, void *statesT, void *statesN, void *hout,
+                      int tail)
 {
+    typedef typename Prod<T>::type P;
     dim3 grid(BH, (D / 16) * (D / 16)), block(64);
+    // chunks in flight per lane when the grid fills the machine: a lane asks for 8 or 16 bytes of products per chunk,
+    // and what hides the latency is the number of bytes on their way
+    constexpr int kFew = sizeof(P) == 2 ? 16 : 4;
     if ((int64_t)grid.y * BH >= 1024) {      // at least a wave per SIMD
-        hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, 4>), grid, block, 0, st, hin, prodT, decay,
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, kFew>), grid, block, 0, st, hin, (const P *)prodT, decay, pexp,
                            (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt);
     } else {
-        hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, 32>), grid, block, 0, st, hin, prodT, decay,
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, 32>), grid, block, 0, st, hin, (const P *)prodT, decay, pexp,
                            (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt);
     }
     return launch_status();
@@ -286,10 +337,10 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const
 
 #define GLA_INST_OUTER(T, C, D, DM)                                                                   \
     template int launch_chunk_outer<T, C, D, DM>(hipStream_t, int, int, int, int, const float *, const void *, \
-                                                 const void *, float *, float *);
+                                                 const void *, void *, float *, unsigned char *);
 #define GLA_INST_SCAN(T, D, DM)                                                                       \
-    template int launch_chunk_scan<T, D, DM>(hipStream_t, int, int, int, int, const void *, const float *, \
-                                             const float *, void *, void *, void *, int);
+    template int launch_chunk_scan<T, D, DM>(hipStream_t, int, int, int, int, const void *, const void *, \
+                                             const float *, const unsigned char *, void *, void *, void *, int);
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUTER)
 GLA_INST_SCAN(__bf16, 32, 16)
 GLA_INST_SCAN(__bf16, 32, 32)

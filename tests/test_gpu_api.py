@@ -113,3 +113,17 @@ def test_chunk_forward_without_gradients_keeps_no_residual():
     assert not hT_b.requires_grad and not out_c.requires_grad
     assert torch.equal(hT_a, hT_b) and torch.equal(out_a, out_b)
     assert torch.equal(hT_a, hT_c) and torch.equal(out_a, out_c)
+
+
+@pytest.mark.parametrize("bad", [float("nan"), float("inf")])
+def test_chunk_values_that_are_not_finite_reach_the_state(bad):
+    """The per-chunk products travel from one kernel to the next as 16-bit mantissas with shared exponents; a
+    product that is not finite must still arrive as such, so that a NaN or an overflow in the inputs shows in
+    hidden_final instead of being swallowed on the way."""
+    from gla_jax_amd import chunk_gla
+    _, dev = gpu_inputs(1, 256, 1, 64, 4.0, seed=17, dtype=torch.bfloat16)
+    dev[2][0, 130, 0, 5] = bad                      # one value of `value`, in the second chunk
+    hT, out = chunk_gla(*dev, 128)
+    assert not torch.isfinite(hT.float()[0, 0, :, 5]).any()          # that value feature of the final state
+    assert torch.isfinite(hT.float()[0, 0, :, 40:]).all()            # value features of other product tiles are untouched
+    assert not torch.isfinite(out.float()[0, 130, 0, 5])
