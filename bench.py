@@ -159,18 +159,20 @@ def bench_chunk(B, T, H, D, chunk, shift, steps, warmup, public=True):
 
     n_th = B * T * H
     N = T // min(chunk, 128)
-    state_f32 = B * H * N * D * D * 4
+    # per-chunk products as the kernels exchange them (16-bit mantissas, an exponent byte per 16 of them) plus
+    # the decays, and one orientation of the chunk states
+    prod = B * H * N * (D * D * 2 + D * D // 16 + D * 4)
     state_bf16 = B * H * N * D * D * 2
     # algorithmic bytes (inputs read once, outputs written once) and what each kernel really moves
     kernels = {
-        "fwd.chunk_outer_kernel": (lambda: fwd(1), 8 * D * n_th, 8 * D * n_th + state_f32),
+        "fwd.chunk_outer_kernel": (lambda: fwd(1), 8 * D * n_th, 8 * D * n_th + prod),
         # the scans write the chunk states in both orientations; the gradient kernel reads three state
         # arrays (S_n, dS' twice) and the gates, q and k a second time (once for the score
         # blocks, once per feature slice; about half of that second read is served by the L2: measured)
-        "fwd.chunk_scan_kernel": (lambda: fwd(2), 0, state_f32 + 2 * state_bf16),
+        "fwd.chunk_scan_kernel": (lambda: fwd(2), 0, prod + 2 * state_bf16),
         "fwd.chunk_out_kernel": (lambda: fwd(4), 12 * D * n_th, 12 * D * n_th + state_bf16),
-        "bwd.chunk_outer_kernel": (lambda: bwd(1), 8 * D * n_th, 8 * D * n_th + state_f32),
-        "bwd.chunk_scan_kernel": (lambda: bwd(2), 0, state_f32 + 2 * state_bf16),
+        "bwd.chunk_outer_kernel": (lambda: bwd(1), 8 * D * n_th, 8 * D * n_th + prod),
+        "bwd.chunk_scan_kernel": (lambda: bwd(2), 0, prod + 2 * state_bf16),
         "bwd.chunk_grad_kernel": (lambda: bwd(4), 22 * D * n_th, 26 * D * n_th + 3 * state_bf16),
     }
     per = {}

@@ -192,8 +192,8 @@ template <typename T> struct Pair;
 template <> struct Pair<__bf16> { typedef bf16x2 type; };
 template <> struct Pair<float> { typedef f32x2 type; };
 
-// U = chunks whose inputs are in flight per thread: 4 when the grid fills the machine, 32 when few (b,h)
-// pairs leave it to the single thread to keep the memory system busy (long sequences, small batch).
+// U = chunks per batch (two batches of inputs are in flight per thread): 8 when the grid fills the machine, 16 when
+// few (b,h) pairs leave it to the single thread to keep the memory system busy (long sequences, small batch).
 // DM: head dimension of hin / hout in memory (16 when D = 32 stands in for it: rows and columns past DM are zero
 // on the way in and are not stored on the way out; the per-chunk buffers are D x D).
 template <typename T, int D, int DM, int U>
@@ -252,40 +252,60 @@ __global__ __launch_bounds__(64) void chunk_scan_kernel(const void *__restrict__
         }
         if (statesN) emit_n(n);
     };
-    auto load_p = [&](int n, f32x4 &pv, float &dc) {
-        if constexpr (sizeof(P) == 4) {
-            pv = *reinterpret_cast<const f32x4 *>(pp + (int64_t)n * D * D);
-        } else {
-            const i16x4 h4 = *reinterpret_cast<const i16x4 *>(pp + (int64_t)n * D * D);
-            const int eb = ep[(int64_t)n * (D * D / 16)];
-            const float sc = eb == kProdNotFinite ? __builtin_nanf("")
-                                                  : __int_as_float((eb + 1) << 23) * (1.f / 32767.f);   // 2^(eb - 126) / 32767
-#pragma unroll
-            for (int e = 0; e < 4; ++e) pv[e] = (float)h4[e] * sc;
-        }
-        dc = dp[(int64_t)n * D];
+    // what a lane asks for per chunk, kept as it arrives until the chunk is worked through (converting it where it
+    // is requested would make the lane wait for it there)
+    struct Raw {
+        typename std::conditional<sizeof(P) == 4, f32x4, i16x4>::type p;
+        int eb;
+        float dc;
     };
-    int step = 0;
-    for (; step + U <= N; step += U) {
-        f32x4 pv[U];
-        float dc[U];
+    auto request = [&](int n, Raw &x) {
+        x.p = *reinterpret_cast<const decltype(x.p) *>(pp + (int64_t)n * D * D);
+        if constexpr (sizeof(P) == 2) x.eb = ep[(int64_t)n * (D * D / 16)];
+        x.dc = dp[(int64_t)n * D];
+    };
+    auto advance = [&](const Raw &x) {
+        if constexpr (sizeof(P) == 4) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) load_p(reverse ? N - 1 - (step + u) : step + u, pv[u], dc[u]);
+            for (int e = 0; e < 4; ++e) X[e] = x.dc * X[e] + x.p[e];
+        } else {
+            const float sc = x.eb == kProdNotFinite ? __builtin_nanf("")
+                                                    : __int_as_float((x.eb + 1) << 23) * (1.f / 32767.f);   // 2^(eb - 126) / 32767
+#pragma unroll
+            for (int e = 0; e < 4; ++e) X[e] = x.dc * X[e] + (float)x.p[e] * sc;
+        }
+    };
+    // Batches of U chunks, the next batch's inputs requested before the current one is worked through: what hides
+    // the latency of the loads is the number of bytes on their way.
+    auto chunk_of = [&](int step) { return reverse ? N - 1 - step : step; };
+    Raw buf[2][U];
+    const int nb = N / U;
+    if (nb > 0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) request(chunk_of(u), buf[0][u]);
+    }
+    auto batch = [&](int b, auto cur, auto nxt) {
+        constexpr int kc = decltype(cur)::value, kn = decltype(nxt)::value;
+        if (b + 1 < nb) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) request(chunk_of((b + 1) * U + u), buf[kn][u]);
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            emit(reverse ? N - 1 - (step + u) : step + u);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) X[e] = dc[u] * X[e] + pv[u][e];
+            emit(chunk_of(b * U + u));
+            advance(buf[kc][u]);
         }
+    };
+    for (int b = 0; b < nb; b += 2) {
+        batch(b, std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
+        if (b + 1 < nb) batch(b + 1, std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
     }
-    for (; step < N; ++step) {
-        const int n = reverse ? N - 1 - step : step;
-        f32x4 pv;
-        float dc;
-        load_p(n, pv, dc);
+    for (int step = nb * U; step < N; ++step) {
+        const int n = chunk_of(step);
+        Raw x;
+        request(n, x);
         emit(n);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) X[e] = dc * X[e] + pv[e];
+        advance(x);
     }
     if (tail && statesN) emit_n(N);
     if (in_mem) store_hidden<4>(hout, hdt, (int64_t)bh * DM * DM + dk * DM + dv0, X);
@@ -322,14 +342,12 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const
 {
     typedef typename Prod<T>::type P;
     dim3 grid(BH, (D / 16) * (D / 16)), block(64);
-    // chunks in flight per lane when the grid fills the machine: a lane asks for 8 or 16 bytes of products per chunk,
-    // and what hides the latency is the number of bytes on their way
-    constexpr int kFew = sizeof(P) == 2 ? 16 : 4;
+    constexpr int kFew = 8;
     if ((int64_t)grid.y * BH >= 1024) {      // at least a wave per SIMD
         hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, kFew>), grid, block, 0, st, hin, (const P *)prodT, decay, pexp,
                            (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt);
     } else {
-        hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, 32>), grid, block, 0, st, hin, (const P *)prodT, decay, pexp,
+        hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, 16>), grid, block, 0, st, hin, (const P *)prodT, decay, pexp,
                            (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt);
     }
     return launch_status();
