@@ -4,6 +4,7 @@ tolerance model of tests/util.py in all seven results.  The cases follow from SW
 names a reproducible case (its index, shape, shift, seeds and resets are printed before anything is launched)
 and another seed is one constant away.  The cases that earlier sweeps found are the named regression tests of
 tests/test_gpu_chunk_regress.py."""
+import os
 import time
 
 import numpy as np
@@ -16,10 +17,11 @@ from tests.util import (check_chunk_outputs, check_recurrent_outputs, cotangents
 
 pytestmark = pytest.mark.gpu
 
-SWEEP_SEED = 31337
-SWEEP_CASES = 150
-SWEEP_SECONDS = 60.0         # stop drawing new cases after this long (at least SWEEP_MIN have run by then)
-SWEEP_MIN = 60
+# GLA_SWEEP_SEED / GLA_SWEEP_CASES in the environment run another or a longer sweep without editing this file
+SWEEP_SEED = int(os.environ.get("GLA_SWEEP_SEED", "31337"))
+SWEEP_CASES = int(os.environ.get("GLA_SWEEP_CASES", "150"))
+SWEEP_SECONDS = 60.0 if "GLA_SWEEP_CASES" not in os.environ else 1e9   # stop drawing new cases after this long
+SWEEP_MIN = min(60, SWEEP_CASES)                                       # ... but not before this many have run
 
 
 def draw_case(rng, it):
