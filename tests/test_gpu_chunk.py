@@ -8,8 +8,8 @@ import torch
 
 from oracle import gla_oracle as O
 from oracle import naive_c
-from tests.util import (GRAD_NAMES, TOL, assert_parity, assert_plain, check_chunk_outputs, cotangents, fmt_log,
-                        gpu_inputs, loss_of, reference_emulation, to_dev, to_np)
+from tests.util import (GRAD_NAMES, TOL, assert_parity, assert_plain, check_chunk_outputs, cotangents, err_over_rms,
+                        fmt_log, gpu_inputs, loss_of, reference_emulation, to_dev, to_np)
 
 pytestmark = pytest.mark.gpu
 
@@ -158,14 +158,27 @@ def _full_shape_check(B, T, H, D, chunk, shift, seed, plain=()):
     exact = naive_c.naive_bwd(h0, g, v, k, q, dhT, dout, dtype=np.float64, nthreads=16)
     log = check_chunk_outputs(dtype, (h0, g, v, k, q), chunk, hT, out, grads, dhT, dout, exact=exact, plain=plain)
     print("max|err|/rms:", fmt_log(log))
+    # what storing the EXACT result in the tensor's own dtype costs: the floor under any implementation's error
+    # (d(log_fgate) is float32: no floor to speak of)
+    names = ("dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery", "hidden_final", "out")
+    floor = {n: err_over_rms(O.bf16_round(np.asarray(e, dtype=np.float32)), e) for n, e in zip(names, exact)
+             if n != "dlog_fgate"}
+    print("storage floor:", {n: f"{x:.2e}" for n, x in floor.items()})
     return log, dev, (hT, out) + tuple(grads), (dhT, dout)
 
 
 def test_chunk_baseline_config_fwd_bwd_full_shape():
-    """BASELINE configs[1]/[2]: B4,T4096,H6,D128, chunk 128, gates log_sigmoid(5+N(0,1)).  Under weak decay the
-    final state and the gradient of the initial one meet the plain north_star bound (no allowance)."""
-    log, _, _, _ = _full_shape_check(4, 4096, 6, 128, 128, 5.0, seed=12, plain=("hidden_final", "dhidden_init"))
-    assert max(a for a, _ in log.values()) <= 3e-2
+    """BASELINE configs[1]/[2]: B4,T4096,H6,D128, chunk 128, gates log_sigmoid(5+N(0,1)), every batch entry and
+    head.  The final state, the gradient of the initial one and d(log_fgate) meet the plain north_star bound
+    (2e-2 RMS, no allowance).  out, dvalue, dkey and dquery do not: storing the exact result in bf16 costs
+    1.3-1.5e-2 there, and eight operand roundings of about 1e-3 RMS each (rescaled q and k, the score blocks, the
+    chunk states) bring the maximum over 12.6 M elements to 2.3-2.5e-2, where the emulated reference sits at
+    3.7-4.1e-2.  They are held to 2.6e-2, a stated gap to the plain bound, not to a blanket allowance."""
+    log, _, _, _ = _full_shape_check(4, 4096, 6, 128, 128, 5.0, seed=12,
+                                     plain=("hidden_final", "dhidden_init", "dlog_fgate"))
+    for name in ("out", "dvalue", "dkey", "dquery"):
+        assert log[name][0] <= 2.6e-2, f"{name}: {log[name][0]:.3e}"
+        assert log[name][0] <= 0.7 * log[name][1], f"{name}: no longer well below the emulated reference"
 
 
 def test_chunk_long_context_strong_decay_full_shape():

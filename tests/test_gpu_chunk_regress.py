@@ -21,7 +21,15 @@ rounding of the score blocks as the operand of dv = A^T dO, under strong decay, 
 carry most of dv.  Those now enter that product (and out = A V in the forward) as bf16 head + remainder.
 
 OPEN_CASES lists cases that are known to fail and not fixed; they are expected failures (strict: a case that
-starts to pass must be moved to SWEEP_CASES).  It is empty."""
+starts to pass must be moved to SWEEP_CASES).  One case: of three further sweeps of 400 cases each (the suite's
+own sweep with other seeds), one found d(log_fgate) of a head-dimension-32 case (one 64-token chunk, three hard
+resets) at 2.35e-2 RMS = 1.63 x the emulated reference (bound 1.5 x).  Per token the gate-cumsum gradient of the
+kernel and of the emulated reference are off by the same amounts (0.1-0.5 in values of 5-150: the bf16 rounding
+of the operands of the dq / dk products); d(log_fgate) is their reverse running sum, a random walk that on these
+inputs ends at +1.1 for the kernel and +0.6 for the reference at the worst token.  With 32 features a sum has a
+quarter of the terms it has at D=128 and the ratio of the two maxima scatters accordingly.  Taking the dyadic
+levels' operand as head + remainder (like the one-anchor path's) changes nothing here and costs the gradient
+kernel spills: not kept."""
 import numpy as np
 import pytest
 import torch
@@ -69,12 +77,15 @@ SWEEP_CASES = {
 
 
 # found by a sweep, out of bounds, not fixed (see the module docstring)
-OPEN_CASES = {}
+OPEN_CASES = {
+    "s202_c342": (1, 64, 4, 32, 32, 5.0, 203242, 342, [55, 13, 23], -200.0, "dlog_fgate"),
+}
 
 
 @pytest.mark.parametrize("case", sorted(SWEEP_CASES) + [
-    pytest.param(c, marks=pytest.mark.xfail(reason="known to be out of bounds, see the module docstring",
-                                            strict=True)) for c in sorted(OPEN_CASES)])
+    pytest.param(c, marks=pytest.mark.xfail(reason="d(log_fgate) 1.63 x the emulated reference (bound 1.5 x), see "
+                                                   "the module docstring", strict=True, raises=AssertionError))
+    for c in sorted(OPEN_CASES)])
 def test_chunk_sweep_case(case):
     from gla_jax_amd import chunk_gla
     B, T, H, D, chunk, shift, seed, cseed, rows, val, _ = {**SWEEP_CASES, **OPEN_CASES}[case]
