@@ -153,7 +153,7 @@ int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments and results as gla_chunk_fwd without the workspace pair: the per-chunk products,
  * decays and chunk-start states go through a static device array of GLA_CHUNK_FWD_STATIC_BYTES bytes
- * (80 MiB: the headline shape B4 T4096 H6 D128 bf16 needs 72.4 MiB) that every GPU the library runs on holds
+ * (80 MiB: the headline shape B4 T4096 H6 D128 bf16 needs 49.1 MiB) that every GPU the library runs on holds
  * from the first call on it until the process ends.  Shapes whose workspace (gla_chunk_fwd_workspace_bytes)
  * exceeds the capacity are rejected with GLA_ERR_WORKSPACE before anything is launched.  The call allocates
  * and frees nothing.  The first call on a device looks up the array's address there (hipGetSymbolAddress):
