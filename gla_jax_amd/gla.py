@@ -339,7 +339,17 @@ def _recurrent(hidden_init, log_fgate, value, key, query, reverse, out_fp32):
     (h0, g, v, k, q), lead, (B, T, H, DK, DV) = _prep(hidden_init, log_fgate, value, key, query)
     if DK != DV:
         raise AssertionError("Not supported yet: key and value head dims differ")      # gla.py:120, 391
+    pad = 16 - DK if DK < 16 else 0
+    if pad:
+        # Head dims below 16 (the reference packs several such heads into one tile, gla.py:60-62): the kernels' smallest
+        # state is 16 x 16, so the rows are padded with zeros here (a zero key, query and value feature with gate 0
+        # leaves the rest of the state and of the output untouched) and the results cut back.
+        F = torch.nn.functional
+        h0 = F.pad(h0, (0, pad, 0, pad))
+        g, v, k, q = (F.pad(x, (0, pad)) for x in (g, v, k, q))
     hT, out = _apply(_RecurrentGLA, h0, g, v, k, q, bool(reverse), bool(out_fp32))
+    if pad:
+        hT, out = hT[..., :DK, :DV], out[..., :DV]
     return _as(hT, lead + (H, DK, DV), hidden_init.dtype), _as(out, lead + (T, H, DV), out.dtype)
 
 

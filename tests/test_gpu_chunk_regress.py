@@ -21,15 +21,25 @@ rounding of the score blocks as the operand of dv = A^T dO, under strong decay, 
 carry most of dv.  Those now enter that product (and out = A V in the forward) as bf16 head + remainder.
 
 OPEN_CASES lists cases that are known to fail and not fixed; they are expected failures (strict: a case that
-starts to pass must be moved to SWEEP_CASES).  One case: of three further sweeps of 400 cases each (the suite's
-own sweep with other seeds), one found d(log_fgate) of a head-dimension-32 case (one 64-token chunk, three hard
+starts to pass must be moved to SWEEP_CASES).  Two cases, of five further sweeps of 400 cases each (the suite's
+own sweep with other seeds).  The first: d(log_fgate) of a head-dimension-32 case (one 64-token chunk, three hard
 resets) at 2.35e-2 RMS = 1.63 x the emulated reference (bound 1.5 x).  Per token the gate-cumsum gradient of the
 kernel and of the emulated reference are off by the same amounts (0.1-0.5 in values of 5-150: the bf16 rounding
 of the operands of the dq / dk products); d(log_fgate) is their reverse running sum, a random walk that on these
 inputs ends at +1.1 for the kernel and +0.6 for the reference at the worst token.  With 32 features a sum has a
 quarter of the terms it has at D=128 and the ratio of the two maxima scatters accordingly.  Taking the dyadic
 levels' operand as head + remainder (like the one-anchor path's) changes nothing here and costs the gradient
-kernel spills: not kept."""
+kernel spills: not kept.
+
+The second: dvalue of a head-dimension-16 case (one 128-token chunk, six resets to -25) at 4.42e-2 RMS = 1.57 x the
+emulated reference.  It is ONE element, ten RMS large: the exact value is 140.389, its bf16 neighbours are 140 and
+141, the emulated reference stores 140 (off by 0.389 = 2.8e-2 RMS, the storage rounding of the exact value) and the
+kernel 141 (off by 0.611): an error of 0.11 before rounding, 0.8e-2 RMS, put the kernel's value past the midpoint.
+Both are neighbours of the exact value; over the whole tensor the kernel's L2 error is 0.85 x the emulated
+reference's (2.99e-3 against 3.51e-3 of an RMS) and with five other cotangents for the same inputs the ratio of the
+maxima is 0.5-0.9.  A bound of 1.5 x the reference's maximum cannot hold against a rounding that falls to the other
+neighbour where the reference's own error on that element is below 0.4 of a spacing; the bound is left as it is and
+the case is listed."""
 import numpy as np
 import pytest
 import torch
@@ -79,12 +89,17 @@ SWEEP_CASES = {
 # found by a sweep, out of bounds, not fixed (see the module docstring)
 OPEN_CASES = {
     "s202_c342": (1, 64, 4, 32, 32, 5.0, 203242, 342, [55, 13, 23], -200.0, "dlog_fgate"),
+    "s404_c360": (2, 128, 2, 16, 32, 5.0, 405260, 360, [102, 57, 35, 46, 68, 56], -25.0, "dvalue"),
+}
+OPEN_REASONS = {
+    "s202_c342": "d(log_fgate) 1.63 x the emulated reference (bound 1.5 x), see the module docstring",
+    "s404_c360": "dvalue 1.57 x the emulated reference (bound 1.5 x): one element stored as the other bf16 neighbour "
+                 "of the exact value, see the module docstring",
 }
 
 
 @pytest.mark.parametrize("case", sorted(SWEEP_CASES) + [
-    pytest.param(c, marks=pytest.mark.xfail(reason="d(log_fgate) 1.63 x the emulated reference (bound 1.5 x), see "
-                                                   "the module docstring", strict=True, raises=AssertionError))
+    pytest.param(c, marks=pytest.mark.xfail(reason=OPEN_REASONS[c], strict=True, raises=AssertionError))
     for c in sorted(OPEN_CASES)])
 def test_chunk_sweep_case(case):
     from gla_jax_amd import chunk_gla

@@ -22,7 +22,7 @@ def run_fwd_bwd(fn, dev, dhT, dout, out_dtype, **kw):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("B,T,H,D", [(2, 67, 3, 64), (1, 32, 2, 16), (1, 40, 1, 128), (2, 24, 2, 32), (3, 1, 5, 64),
-                                     (1, 17, 1, 64), (2, 45, 2, 256)])
+                                     (1, 17, 1, 64), (2, 45, 2, 256), (2, 37, 3, 8), (1, 20, 2, 4)])
 @pytest.mark.parametrize("reverse", [False, True])
 def test_recurrent_gla_matches_oracle(dtype, B, T, H, D, reverse):
     from gla_jax_amd import recurrent_gla
