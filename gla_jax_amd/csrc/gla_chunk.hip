@@ -15,6 +15,22 @@ struct ChunkPlan {
     size_t prod = 0, decay = 0, states = 0;   // byte sizes, each rounded up to 256
     size_t scale_off = 0;                     // where the products' exponents start inside the decay region
     size_t resid = 0;                         // the forward residual: N + 1 states per (b,h), the last one final
+    // Head dimension 256 runs as two passes of the 128-feature kernels over 2H heads (gla_chunk_split.hip); the
+    // sizes above are then those of one such pass, and:
+    bool split = false;
+    size_t rows = 0;                          // one [B,T,H,256] array of the element type
+    size_t rows_f32 = 0;                      // ... of floats
+    size_t hid = 0;                           // one [B,2H,128,128] array of states (sized for fp32 states)
+    bool wide = false;                        // bf16 data: both passes leave their results in fp32, summed and rounded once
+    // forward: value rows with their halves exchanged, the second pass's out (fp32 data) or both passes' (bf16 data),
+    // hidden_init and hidden_final in blocks; backward: value and dout rows exchanged, the second pass's dq, dk, dv
+    // (or both passes'), its d(log_fgate), the states' cotangents in blocks
+    size_t fwd_bytes() const { return prod + decay + states + (split ? rows + (wide ? 2 : 1) * rows_f32 + 4 * hid : 0); }
+    size_t bwd_bytes() const
+    {
+        return prod + decay + 2 * states + (split ? 2 * rows + (wide ? 7 : 4) * rows_f32 + 4 * hid : 0);
+    }
+    size_t resid_bytes() const { return split ? 2 * resid : resid; }
 };
 
 static size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -34,8 +50,18 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
     if (DK != DV) return GLA_ERR_SHAPE;                      // gla.py:499
     if (!is_pow2(chunk) || T % chunk != 0) return GLA_ERR_CHUNK;   // gla.py:500, 674
     if (chunk < 32) return GLA_ERR_UNSUPPORTED;
-    // largest tile built: 128 tokens for bf16 (32 at D=256), for fp32 (tiles twice as wide) 64 at D<=64 and 32 at D=128
-    int64_t C = dtype == GLA_BF16 ? (DK > 128 ? 32 : 128) : (DK > 64 ? 32 : 64);
+    if (DK == 256) {
+        int rc = plan_chunk(B, T, 2 * H, 128, 128, chunk, dtype, plan, hidden_dtype);
+        if (rc) return rc;
+        plan->split = true;
+        plan->wide = dtype == GLA_BF16;
+        plan->rows = round256((size_t)B * T * H * 256 * (dtype == GLA_BF16 ? 2 : 4));
+        plan->rows_f32 = round256((size_t)B * T * H * 256 * sizeof(float));
+        plan->hid = round256((size_t)B * 2 * H * 128 * 128 * sizeof(float));
+        return GLA_OK;
+    }
+    // largest tile built: 128 tokens for bf16, for fp32 (tiles twice as wide) 64 at D<=64 and 32 at D=128
+    int64_t C = dtype == GLA_BF16 ? 128 : (DK > 64 ? 32 : 64);
     while (T % C != 0) C /= 2;                               // chunk >= 32 divides T, so this stops at 32 or above
     int Dk = 0;
 #define GLA_PLAN_CASE(T_, C_, D_, DM_) \
@@ -106,7 +132,7 @@ extern "C" size_t gla_chunk_states_bytes(int64_t B, int64_t T, int64_t H, int64_
                                          int64_t chunk_size, gla_dtype dtype)
 {
     ChunkPlan p;
-    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.resid : 0;
+    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.resid_bytes() : 0;
 }
 
 extern "C" size_t gla_chunk_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
@@ -114,7 +140,7 @@ extern "C" size_t gla_chunk_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H,
 {
     ChunkPlan p;
     // per-chunk products, decays, and the chunk-start states in [dv][dk] orientation for the output kernel
-    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.prod + p.decay + p.states : 0;
+    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.fwd_bytes() : 0;
 }
 
 extern "C" size_t gla_chunk_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
@@ -122,15 +148,15 @@ extern "C" size_t gla_chunk_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H,
 {
     ChunkPlan p;
     // per-chunk products, decays, and d(chunk-end state) in both orientations
-    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.prod + p.decay + 2 * p.states : 0;
+    return plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p) == GLA_OK ? p.bwd_bytes() : 0;
 }
 
-extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK,
-                                    int64_t DV, int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
-                                    const void *hidden_init,
-                                    const float *log_fgate, const void *value, const void *key,
-                                    const void *query, void *hidden_final, void *out, void *states,
-                                    void *workspace, size_t workspace_bytes)
+// wide != 0 (bf16 data at head dimension 128 only): `out` is a float array
+static int chunk_fwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                         int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype, const void *hidden_init,
+                         const float *log_fgate, const void *value, const void *key, const void *query,
+                         void *hidden_final, void *out, void *states, void *workspace, size_t workspace_bytes,
+                         int wide)
 {
     ChunkPlan p;
     int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p, hidden_dtype);
@@ -140,9 +166,36 @@ extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t
         if (!ptr) return GLA_ERR_NULL;
         if (!aligned16(ptr)) return GLA_ERR_ALIGN;
     }
-    if (!workspace || workspace_bytes < p.prod + p.decay + p.states) return GLA_ERR_WORKSPACE;
+    if (!workspace || workspace_bytes < p.fwd_bytes()) return GLA_ERR_WORKSPACE;
     if (!aligned16(workspace) || (states && !aligned16(states))) return GLA_ERR_ALIGN;
     unsigned char *ws = (unsigned char *)workspace;
+    if (p.split) {
+        // Two passes of the 128-feature kernels over 2H heads: key half a with value half a on the arrays as they
+        // lie, then key half a with the other value half (value rows with their halves exchanged); the second
+        // pass's outputs belong to the other half of each row and are added there.
+        if (stages != 7) return GLA_ERR_UNSUPPORTED;
+        hipStream_t st = (hipStream_t)stream;
+        const size_t sub = p.prod + p.decay + p.states;
+        if (wide) return GLA_ERR_UNSUPPORTED;
+        unsigned char *v_sw = ws + sub, *out2 = v_sw + p.rows, *out1 = out2 + p.rows_f32,
+                      *h0_same = out2 + (p.wide ? 2 : 1) * p.rows_f32, *h0_cross = h0_same + p.hid,
+                      *hT_same = h0_cross + p.hid, *hT_cross = hT_same + p.hid;
+        int e = launch_hidden_blocks(st, hidden_dtype, B * H, const_cast<void *>(hidden_init), h0_same, h0_cross, 1);
+        if (e) return e;
+        e = launch_swap_halves(st, dtype, B * T * H, v_sw, value);
+        if (e) return e;
+        e = chunk_fwd_run(stream, 7, B, T, 2 * H, 128, 128, chunk_size, dtype, hidden_dtype, h0_same, log_fgate, value,
+                          key, query, hT_same, p.wide ? (void *)out1 : out, states, ws, sub, p.wide);
+        if (e) return e;
+        e = chunk_fwd_run(stream, 7, B, T, 2 * H, 128, 128, chunk_size, dtype, hidden_dtype, h0_cross, log_fgate, v_sw,
+                          key, query, hT_cross, out2, states ? (unsigned char *)states + p.resid : nullptr, ws, sub,
+                          p.wide);
+        if (e) return e;
+        e = p.wide ? launch_sum_rows(st, B * T * H, out, (const float *)out1, (const float *)out2, 1)
+                   : launch_add_rows(st, dtype, B * T * H, out, out2, 1);
+        if (e) return e;
+        return launch_hidden_blocks(st, hidden_dtype, B * H, hidden_final, hT_same, hT_cross, 0);
+    }
     void *prodT = (void *)ws;
     float *decay = (float *)(ws + p.prod);
     unsigned char *pexp = ws + p.prod + p.scale_off;
@@ -161,11 +214,29 @@ extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t
             e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 0, hidden_dtype, hidden_init, prodT, decay, pexp,
                                               statesT, states, hidden_final, 1);
         if (e) return e;
-        if (stages & 4)
+        if ((stages & 4) && !wide)
             e = launch_chunk_out<E, C_, D_, DM_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, statesT,
                                                  out);
+        if ((stages & 4) && wide) {
+            if constexpr (sizeof(E) == 2 && D_ == 128 && DM_ == 128)
+                e = launch_chunk_out<E, C_, D_, DM_, true>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query,
+                                                           statesT, out);
+            else
+                e = GLA_ERR_UNSUPPORTED;
+        }
         return e;
     });
+}
+
+extern "C" int gla_chunk_fwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK,
+                                    int64_t DV, int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
+                                    const void *hidden_init,
+                                    const float *log_fgate, const void *value, const void *key,
+                                    const void *query, void *hidden_final, void *out, void *states,
+                                    void *workspace, size_t workspace_bytes)
+{
+    return chunk_fwd_run(stream, stages, B, T, H, DK, DV, chunk_size, dtype, hidden_dtype, hidden_init, log_fgate,
+                         value, key, query, hidden_final, out, states, workspace, workspace_bytes, 0);
 }
 
 extern "C" int gla_chunk_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
@@ -187,7 +258,7 @@ extern "C" int gla_chunk_fwd_static(void *stream, int64_t B, int64_t T, int64_t 
     ChunkPlan p;
     int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p, hidden_dtype);
     if (rc) return rc;
-    if (p.prod + p.decay + p.states > kStaticScratchBytes) return GLA_ERR_WORKSPACE;   // beyond the static array
+    if (p.fwd_bytes() > kStaticScratchBytes) return GLA_ERR_WORKSPACE;   // beyond the static array
     void *ws = nullptr;
     rc = static_scratch(&ws);
     if (rc) return rc;
@@ -197,13 +268,12 @@ extern "C" int gla_chunk_fwd_static(void *stream, int64_t B, int64_t T, int64_t 
                                 value, key, query, hidden_final, out, states, ws, kStaticScratchBytes);
 }
 
-extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK,
-                                    int64_t DV, int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
-                                    const float *log_fgate,
-                                    const void *value, const void *key, const void *query, const void *states,
-                                    const void *dhidden_final, const void *dout, void *dhidden_init,
-                                    float *dlog_fgate, void *dvalue, void *dkey, void *dquery,
-                                    void *workspace, size_t workspace_bytes)
+// wide != 0 (bf16 data at head dimension 128 only): `dvalue`, `dkey`, `dquery` are float arrays
+static int chunk_bwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                         int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype, const float *log_fgate,
+                         const void *value, const void *key, const void *query, const void *states,
+                         const void *dhidden_final, const void *dout, void *dhidden_init, float *dlog_fgate,
+                         void *dvalue, void *dkey, void *dquery, void *workspace, size_t workspace_bytes, int wide)
 {
     ChunkPlan p;
     int rc = plan_chunk(B, T, H, DK, DV, chunk_size, dtype, &p, hidden_dtype);
@@ -214,9 +284,55 @@ extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t
         if (!ptr) return GLA_ERR_NULL;
         if (!aligned16(ptr)) return GLA_ERR_ALIGN;
     }
-    if (!workspace || workspace_bytes < p.prod + p.decay + 2 * p.states) return GLA_ERR_WORKSPACE;
+    if (!workspace || workspace_bytes < p.bwd_bytes()) return GLA_ERR_WORKSPACE;
     if (!aligned16(workspace)) return GLA_ERR_ALIGN;
     unsigned char *ws = (unsigned char *)workspace;
+    if (p.split) {
+        // The two passes of the forward again: the first writes its gradients into the caller's arrays, the second
+        // into the workspace, from where they are added (those of the value side to the other half of each row).
+        if (stages != 7) return GLA_ERR_UNSUPPORTED;
+        hipStream_t st = (hipStream_t)stream;
+        const size_t sub = p.prod + p.decay + 2 * p.states;
+        if (wide) return GLA_ERR_UNSUPPORTED;
+        unsigned char *v_sw = ws + sub, *do_sw = v_sw + p.rows, *dg2 = do_sw + p.rows, *dq2 = dg2 + p.rows_f32,
+                      *dk2 = dq2 + p.rows_f32, *dv2 = dk2 + p.rows_f32, *dq1 = dv2 + p.rows_f32,
+                      *dk1 = dq1 + p.rows_f32, *dv1 = dk1 + p.rows_f32,
+                      *dhT_same = dv2 + (p.wide ? 4 : 1) * p.rows_f32, *dhT_cross = dhT_same + p.hid,
+                      *dh0_same = dhT_cross + p.hid, *dh0_cross = dh0_same + p.hid;
+        const int64_t rows = B * T * H;
+        int e = launch_hidden_blocks(st, hidden_dtype, B * H, const_cast<void *>(dhidden_final), dhT_same, dhT_cross, 1);
+        if (e) return e;
+        e = launch_swap_halves(st, dtype, rows, v_sw, value);
+        if (e) return e;
+        e = launch_swap_halves(st, dtype, rows, do_sw, dout);
+        if (e) return e;
+        e = chunk_bwd_run(stream, 7, B, T, 2 * H, 128, 128, chunk_size, dtype, hidden_dtype, log_fgate, value, key,
+                          query, states, dhT_same, dout, dh0_same, dlog_fgate, p.wide ? (void *)dv1 : dvalue,
+                          p.wide ? (void *)dk1 : dkey, p.wide ? (void *)dq1 : dquery, ws, sub, p.wide);
+        if (e) return e;
+        e = chunk_bwd_run(stream, 7, B, T, 2 * H, 128, 128, chunk_size, dtype, hidden_dtype, log_fgate, v_sw, key, query,
+                          (const unsigned char *)states + p.resid, dhT_cross, do_sw, dh0_cross, (float *)dg2, dv2, dk2,
+                          dq2, ws, sub, p.wide);
+        if (e) return e;
+        if (p.wide) {
+            e = launch_sum_rows(st, rows, dquery, (const float *)dq1, (const float *)dq2, 0);
+            if (e) return e;
+            e = launch_sum_rows(st, rows, dkey, (const float *)dk1, (const float *)dk2, 0);
+            if (e) return e;
+            e = launch_sum_rows(st, rows, dvalue, (const float *)dv1, (const float *)dv2, 1);
+            if (e) return e;
+        } else {
+            e = launch_add_rows(st, dtype, rows, dquery, dq2, 0);
+            if (e) return e;
+            e = launch_add_rows(st, dtype, rows, dkey, dk2, 0);
+            if (e) return e;
+            e = launch_add_rows(st, dtype, rows, dvalue, dv2, 1);
+            if (e) return e;
+        }
+        e = launch_add_rows(st, GLA_F32, rows, dlog_fgate, dg2, 0);
+        if (e) return e;
+        return launch_hidden_blocks(st, hidden_dtype, B * H, dhidden_init, dh0_same, dh0_cross, 0);
+    }
     void *prodT = (void *)ws;
     float *decay = (float *)(ws + p.prod);
     unsigned char *pexp = ws + p.prod + p.scale_off;
@@ -236,11 +352,32 @@ extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t
             e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 1, hidden_dtype, dhidden_final, prodT, decay, pexp,
                                               dstatesT, dstatesN, dhidden_init, 0);
         if (e) return e;
-        if (stages & 4)
+        if ((stages & 4) && !wide)
             e = launch_chunk_grad<E, C_, D_, DM_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,
                                                   states, dstatesT, dstatesN, dlog_fgate, dvalue, dkey, dquery);
+        if ((stages & 4) && wide) {
+            if constexpr (sizeof(E) == 2 && D_ == 128 && DM_ == 128)
+                e = launch_chunk_grad<E, C_, D_, DM_, true>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query,
+                                                            dout, states, dstatesT, dstatesN, dlog_fgate, dvalue, dkey,
+                                                            dquery);
+            else
+                e = GLA_ERR_UNSUPPORTED;
+        }
         return e;
     });
+}
+
+extern "C" int gla_chunk_bwd_stages(void *stream, int stages, int64_t B, int64_t T, int64_t H, int64_t DK,
+                                    int64_t DV, int64_t chunk_size, gla_dtype dtype, gla_dtype hidden_dtype,
+                                    const float *log_fgate,
+                                    const void *value, const void *key, const void *query, const void *states,
+                                    const void *dhidden_final, const void *dout, void *dhidden_init,
+                                    float *dlog_fgate, void *dvalue, void *dkey, void *dquery,
+                                    void *workspace, size_t workspace_bytes)
+{
+    return chunk_bwd_run(stream, stages, B, T, H, DK, DV, chunk_size, dtype, hidden_dtype, log_fgate, value, key, query,
+                         states, dhidden_final, dout, dhidden_init, dlog_fgate, dvalue, dkey, dquery, workspace,
+                         workspace_bytes, 0);
 }
 
 extern "C" int gla_chunk_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,

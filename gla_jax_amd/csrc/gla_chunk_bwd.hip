@@ -33,13 +33,17 @@
 
 namespace gla {
 
-template <typename T, int C, int D, int DM>
+// WIDE: dv, dk and dq are float arrays (the sums of two such runs are rounded once: head dimension 256,
+// gla_chunk_split.hip).
+template <typename T, int C, int D, int DM, bool WIDE>
 __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k,
     const T *__restrict__ q, const T *__restrict__ dout, const T *__restrict__ statesN,
     const T *__restrict__ dstatesT, const T *__restrict__ dstatesN, float *__restrict__ dg,
-    T *__restrict__ dv, T *__restrict__ dk, T *__restrict__ dq, int T_len, int H)
+    std::conditional_t<WIDE, float, T> *__restrict__ dv, std::conditional_t<WIDE, float, T> *__restrict__ dk,
+    std::conditional_t<WIDE, float, T> *__restrict__ dq, int T_len, int H)
 {
+    typedef std::conditional_t<WIDE, float, T> TG;      // element type of dv, dk, dq
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4;
     constexpr int LS = TileGeom<T, D>::kStride;
     constexpr int XS = 32 + 16 / (int)sizeof(T);   // row stride of the per-wave slice scratch
@@ -522,7 +526,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 o[e] = fast_exp2(p8[e]) * hacc + dq8[e];
                 dl8[e] += qr[e] * hacc;
             }
-            st8_row_once<D, DM>(dq + rowoff + fo, c, pack8<T>(o));
+            st8_row_once<D, DM>(dq + rowoff + fo, c, pack8<TG>(o));
         }
         // -- dk: state term V dS'^T first, then the later sub-blocks in descending order
         {
@@ -567,7 +571,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 o[e] = fast_exp2(s8[e]) * hacc + dk8[e];
                 dl8[e] -= krt[e] * hacc;
             }
-            st8_row_once<D, DM>(dk + rowoff + fo, c, pack8<T>(o));
+            st8_row_once<D, DM>(dk + rowoff + fo, c, pack8<TG>(o));
         }
         // -- dv: state term K~ dS' first, then the own and the later sub-blocks
         {
@@ -595,7 +599,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             float o[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
-            st8_row_once<D, DM>(dv + rowoff + fo, c, pack8<T>(o));
+            st8_row_once<D, DM>(dv + rowoff + fo, c, pack8<TG>(o));
         }
         // -- dL of the slice is complete: reverse cumsum inside the sub-block (gla.py:616-617), then, once
         // every wave has published its sub-block total, over the whole chunk + the chunk-level term (gla.py:782)
@@ -636,7 +640,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     }
 }
 
-template <typename T, int C, int D, int DM>
+template <typename T, int C, int D, int DM, bool WIDE>
 int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
                       const void *q, const void *dout, const void *statesN, const void *dstatesT,
                       const void *dstatesN, float *dg, void *dv, void *dk, void *dq)
@@ -648,20 +652,25 @@ int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, c
     const size_t lds = ((size_t)(3 * C + VR) * LS + (size_t)NB * 16 * XS) * sizeof(T) +
                        ((size_t)(3 * NB + 1) * D + NB * 32) * sizeof(float) +
                        ((C - 96) * LS >= NB * 16 * 32 || sizeof(T) != 2 ? 0 : (size_t)NB * 16 * 32 * sizeof(T));
-    auto kern = chunk_grad_kernel<T, C, D, DM>;
+    auto kern = chunk_grad_kernel<T, C, D, DM, WIDE>;
+    typedef std::conditional_t<WIDE, float, T> TG;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(T_len / C * H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
                        (const T *)dout, (const T *)statesN, (const T *)dstatesT, (const T *)dstatesN, dg,
-                       (T *)dv, (T *)dk, (T *)dq, T_len, H);
+                       (TG *)dv, (TG *)dk, (TG *)dq, T_len, H);
     return launch_status();
 }
 
-#define GLA_INST_GRAD(T, C, D, DM)                                                                       \
-    template int launch_chunk_grad<T, C, D, DM>(hipStream_t, int, int, int, const float *, const void *, \
-                                                const void *, const void *, const void *, const void *, \
-                                                const void *, const void *, float *, void *, void *, void *);
+#define GLA_INST_GRAD_AS(T, C, D, DM, WIDE)                                                                    \
+    template int launch_chunk_grad<T, C, D, DM, WIDE>(hipStream_t, int, int, int, const float *, const void *, \
+                                                      const void *, const void *, const void *, const void *, \
+                                                      const void *, const void *, float *, void *, void *, void *);
+#define GLA_INST_GRAD(T, C, D, DM) GLA_INST_GRAD_AS(T, C, D, DM, false)
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_GRAD)
+GLA_INST_GRAD_AS(__bf16, 128, 128, 128, true)
+GLA_INST_GRAD_AS(__bf16, 64, 128, 128, true)
+GLA_INST_GRAD_AS(__bf16, 32, 128, 128, true)
 
 }  // namespace gla

@@ -22,10 +22,11 @@ namespace gla {
 // Resources: two tiles (keys of all but the last sub-block, values), 32 staged state rows and a table
 // fit twice into a CU's LDS, and the register budget is held to what lets two workgroups share a CU, so
 // that one loads while the other computes.
-template <typename T, int C, int D, int DM>
+// WIDE: `out` is a float array (the sum of two such runs is rounded once: head dimension 256, gla_chunk_split.hip).
+template <typename T, int C, int D, int DM, bool WIDE>
 __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C / 32))) void chunk_out_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k, const T *__restrict__ q,
-    const T *__restrict__ states, T *__restrict__ out, int T_len, int H)
+    const T *__restrict__ states, std::conditional_t<WIDE, float, T> *__restrict__ out, int T_len, int H)
 {
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4;
     constexpr int LS = TileGeom<T, D>::kStride;
@@ -169,7 +170,7 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
         float o[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
-        st8_row_once<D, DM>(out + rowoff + fo, c, pack8<T>(o));
+        st8_row_once<D, DM>(out + rowoff + fo, c, pack8<std::conditional_t<WIDE, float, T>>(o));
         if (ks + 1 < KS) {
             __syncthreads();             // every wave is done with the staged rows
             stage_store();
@@ -179,24 +180,28 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     }
 }
 
-template <typename T, int C, int D, int DM>
+template <typename T, int C, int D, int DM, bool WIDE>
 int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
                      const void *q, const void *states, void *out)
 {
     constexpr int LS = TileGeom<T, D>::kStride;
     const size_t lds = (size_t)(2 * C - 16 + 32) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
-    auto kern = chunk_out_kernel<T, C, D, DM>;
+    auto kern = chunk_out_kernel<T, C, D, DM, WIDE>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(T_len / C * H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
-                       (const T *)states, (T *)out, T_len, H);
+                       (const T *)states, (std::conditional_t<WIDE, float, T> *)out, T_len, H);
     return launch_status();
 }
 
-#define GLA_INST_OUT(T, C, D, DM)                                                                      \
-    template int launch_chunk_out<T, C, D, DM>(hipStream_t, int, int, int, const float *, const void *, \
-                                               const void *, const void *, const void *, void *);
+#define GLA_INST_OUT_AS(T, C, D, DM, WIDE)                                                                   \
+    template int launch_chunk_out<T, C, D, DM, WIDE>(hipStream_t, int, int, int, const float *, const void *, \
+                                                     const void *, const void *, const void *, void *);
+#define GLA_INST_OUT(T, C, D, DM) GLA_INST_OUT_AS(T, C, D, DM, false)
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUT)
+GLA_INST_OUT_AS(__bf16, 128, 128, 128, true)
+GLA_INST_OUT_AS(__bf16, 64, 128, 128, true)
+GLA_INST_OUT_AS(__bf16, 32, 128, 128, true)
 
 }  // namespace gla

@@ -65,14 +65,25 @@ def test_chunk_plan_and_sizes():
     assert lib.gla_chunk_states_bytes(B, T, H, 128, 64, 128, _lib.GLA_BF16) == 0  # DK != DV
     # fp32 at D=128 runs on the 32-token tile: 4x as many chunks, 4-byte elements
     assert lib.gla_chunk_states_bytes(B, T, H, D, D, 128, _lib.GLA_F32) == B * H * (4 * n_chunks + 1) * D * D * 4
-    # head dims built: 32, 64, 128, and 256 on 32-token tiles for bf16 only (fp32 tiles are twice as wide)
+    # head dims built: 32, 64, 128; 256 runs as two passes of the 128-feature kernels over twice the heads
     assert lib.gla_chunk_states_bytes(B, T, H, 32, 32, 128, _lib.GLA_BF16) == B * H * (n_chunks + 1) * 32 * 32 * 2
     assert lib.gla_chunk_states_bytes(B, T, H, 32, 32, 128, _lib.GLA_F32) == B * H * (2 * n_chunks + 1) * 32 * 32 * 4
     # head dim 16 runs on the 32-feature kernels: the library's own buffers are sized for 32 x 32 states
     assert lib.gla_chunk_states_bytes(B, T, H, 16, 16, 128, _lib.GLA_BF16) == B * H * (n_chunks + 1) * 32 * 32 * 2
     assert lib.gla_chunk_states_bytes(B, T, H, 8, 8, 128, _lib.GLA_BF16) == 0
-    assert lib.gla_chunk_states_bytes(B, T, H, 256, 256, 128, _lib.GLA_BF16) == B * H * (4 * n_chunks + 1) * 256 * 256 * 2
-    assert lib.gla_chunk_states_bytes(B, T, H, 256, 256, 128, _lib.GLA_F32) == 0
+    assert lib.gla_chunk_states_bytes(B, T, H, 256, 256, 128, _lib.GLA_BF16) == 2 * lib.gla_chunk_states_bytes(
+        B, T, 2 * H, 128, 128, 128, _lib.GLA_BF16) == B * H * (n_chunks + 1) * 256 * 256 * 2
+    assert lib.gla_chunk_states_bytes(B, T, H, 256, 256, 128, _lib.GLA_F32) == B * H * (4 * n_chunks + 1) * 256 * 256 * 4
+    # its workspace: one pass's, the value-side arrays with their halves exchanged, both passes' results in fp32
+    # (out; dq, dk, dv, and the second pass's d(log_fgate)) and the states cut into blocks
+    rows = B * T * H * 256 * 2
+    hid = 4 * B * H * 256 * 256 * 2
+    sub = lib.gla_chunk_fwd_workspace_bytes(B, T, 2 * H, 128, 128, 128, _lib.GLA_BF16)
+    assert sub + 5 * rows + hid <= lib.gla_chunk_fwd_workspace_bytes(B, T, H, 256, 256, 128, _lib.GLA_BF16) <= (
+        sub + 5 * rows + hid + 8 * 256)
+    sub = lib.gla_chunk_bwd_workspace_bytes(B, T, 2 * H, 128, 128, 128, _lib.GLA_BF16)
+    assert sub + 16 * rows + hid <= lib.gla_chunk_bwd_workspace_bytes(B, T, H, 256, 256, 128, _lib.GLA_BF16) <= (
+        sub + 16 * rows + hid + 12 * 256)
     assert lib.gla_chunk_states_bytes(B, T, H, 512, 512, 128, _lib.GLA_BF16) == 0
 
 

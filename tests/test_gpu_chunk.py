@@ -30,8 +30,10 @@ CASES = [
     (torch.float32, 1, 256, 2, 128, 128, 4.0),      # fp32 at D=128 runs on the 32-token tile
     (torch.bfloat16, 3, 128, 5, 128, 128, 3.0),     # a single chunk per sequence, odd batch and head counts
     (torch.bfloat16, 1, 64, 1, 64, 64, 3.0),
-    (torch.bfloat16, 2, 160, 2, 256, 32, 4.0),      # head dimension 256 (32-token tiles)
+    (torch.bfloat16, 2, 160, 2, 256, 32, 4.0),      # head dimension 256: four problems of head dimension 128
     (torch.bfloat16, 1, 256, 1, 256, 128, 0.0),     # the same under strong decay
+    (torch.bfloat16, 2, 384, 3, 256, 128, 2.0),
+    (torch.float32, 2, 96, 2, 256, 32, 3.0),        # ... and in fp32
     (torch.bfloat16, 2, 256, 3, 32, 128, 3.0),      # head dimension 32: one k-step per feature contraction
     (torch.bfloat16, 1, 192, 2, 32, 64, 0.0),       # ... 64-token tiles, strong decay
     (torch.bfloat16, 1, 96, 1, 32, 32, 5.0),        # ... 32-token tiles
@@ -140,9 +142,9 @@ def test_chunk_rejects_what_the_reference_rejects():
         chunk_gla(*dev, 64)                 # 96 % 64 != 0 (einops rearrange, gla.py:674)
     with pytest.raises(_lib.GlaError):
         chunk_gla(*dev, 8)                  # below the smallest tile built here
-    (_, _, _, _, _), dev = gpu_inputs(1, 64, 1, 256, 2.0, seed=3, dtype=torch.float32)
+    (_, _, _, _, _), dev = gpu_inputs(1, 64, 1, 512, 2.0, seed=3, dtype=torch.float32)
     with pytest.raises(_lib.GlaError):
-        chunk_gla(*dev, 32)                 # fp32 at head dimension 256: its tiles do not fit a CU's LDS
+        chunk_gla(*dev, 32)                 # head dimensions above 256 are not built
 
 
 def _full_shape_check(B, T, H, D, chunk, shift, seed, plain=()):

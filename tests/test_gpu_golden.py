@@ -50,14 +50,15 @@ def test_recurrent_gla_against_golden(dtype, reverse):
     check_recurrent_outputs(dtype, golden(d, "rev" if reverse else "fwd"), hT, out, grads)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("reverse", [False, True])
-def test_recurrent_gla_small_head_dim_against_golden(reverse):
-    """Head dim 8 is below what the kernels are built for: the front-end must refuse it, not fall back."""
+def test_recurrent_gla_small_head_dim_against_golden(dtype, reverse):
+    """Head dim 8 is below the kernels' smallest state: the front-end pads the rows to 16 and cuts the results back."""
     from gla_jax_amd import recurrent_gla
     d = load("gla_T12_H2_D8.npz")
-    from gla_jax_amd._lib import GlaError
-    with pytest.raises(GlaError):
-        recurrent_gla(*device_inputs(d, torch.float32), reverse=reverse)
+    hT, out, grads = fwd_bwd(recurrent_gla, d, dtype, reverse=reverse)
+    assert out.shape[-1] == 8 and hT.shape[-2:] == (8, 8)
+    check_recurrent_outputs(dtype, golden(d, "rev" if reverse else "fwd"), hT, out, grads)
 
 
 def test_scans_against_golden():

@@ -3,7 +3,8 @@ types, every head dimension and tile, both directions, gate shifts -2..5, scatte
 tolerance model of tests/util.py in all seven results.  The cases follow from SWEEP_SEED alone, so a failure
 names a reproducible case (its index, shape, shift, seeds and resets are printed before anything is launched)
 and another seed is one constant away.  The cases that earlier sweeps found are the named regression tests of
-tests/test_gpu_chunk_regress.py."""
+tests/test_gpu_chunk_regress.py; a case of THIS sweep that is out of bounds and not fixed is listed there as an
+expected failure and here in KNOWN_OPEN: the sweep still runs it and fails if it has started to pass."""
 import os
 import time
 
@@ -22,6 +23,8 @@ SWEEP_SEED = int(os.environ.get("GLA_SWEEP_SEED", "31337"))
 SWEEP_CASES = int(os.environ.get("GLA_SWEEP_CASES", "150"))
 SWEEP_SECONDS = 60.0 if "GLA_SWEEP_CASES" not in os.environ else 1e9   # stop drawing new cases after this long
 SWEEP_MIN = min(60, SWEEP_CASES)                                       # ... but not before this many have run
+# (seed, case index) -> its name in OPEN_CASES of tests/test_gpu_chunk_regress.py
+KNOWN_OPEN = {(31337, 43): "s31337_c43"}
 
 
 def draw_case(rng, it):
@@ -30,7 +33,7 @@ def draw_case(rng, it):
     B, H = int(rng.integers(1, 4)), int(rng.integers(1, 5))
     shift = float(rng.choice([-2.0, 0.0, 1.0, 3.0, 5.0]))
     if kind == "chunk":
-        D = int(rng.choice([16, 32, 64, 128, 128, 256])) if dtype == torch.bfloat16 else int(rng.choice([16, 32, 64, 128]))
+        D = int(rng.choice([16, 32, 64, 128, 128, 256])) if dtype == torch.bfloat16 else int(rng.choice([16, 32, 64, 128, 256]))
         chunk = int(rng.choice([32, 64, 128]))
         T = chunk * int(rng.integers(1, 5))
         reverse = False
@@ -75,6 +78,12 @@ def test_randomized_sweep():
         if done >= SWEEP_MIN and time.time() - t0 > SWEEP_SECONDS:
             break
         print(f"sweep seed {SWEEP_SEED} case {it}: {c}", flush=True)
+        if (SWEEP_SEED, it) in KNOWN_OPEN:
+            with pytest.raises(AssertionError):
+                run_case(c)
+            print(f"  known open case {KNOWN_OPEN[(SWEEP_SEED, it)]}: still out of bounds")
+            done += 1
+            continue
         log = run_case(c)                    # raises on the first tensor out of bounds: the line above names the case
         done += 1
         for name, (a, b) in log.items():
