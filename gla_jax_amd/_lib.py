@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgla_hip.so")
 
 GLA_F32, GLA_BF16 = 0, 1
-ABI_VERSION = 2                             # GLA_HIP_ABI_VERSION of include/gla_hip.h
+ABI_VERSION = 3                             # GLA_HIP_ABI_VERSION of include/gla_hip.h
 GLA_CHUNK_FWD_STATIC_BYTES = 80 << 20      # capacity of gla_chunk_fwd_static's workspace (gla_hip.h)
 
 _i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
@@ -24,6 +24,10 @@ SIGNATURES = {
     "gla_rnn_scan_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int]),
     "gla_recurrent_fwd": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _int] + [_vp] * 7),
     "gla_recurrent_bwd": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _int] + [_vp] * 13),
+    "gla_recurrent_fwd_workspace_bytes": (_sz, [_i64] * 5 + [_int]),
+    "gla_recurrent_bwd_workspace_bytes": (_sz, [_i64] * 5 + [_int]),
+    "gla_recurrent_fwd_ws": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _int] + [_vp] * 8 + [_sz]),
+    "gla_recurrent_bwd_ws": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _int] + [_vp] * 14 + [_sz]),
     "gla_chunk_states_bytes": (_sz, [_i64] * 6 + [_int]),
     "gla_chunk_fwd_workspace_bytes": (_sz, [_i64] * 6 + [_int]),
     "gla_chunk_bwd_workspace_bytes": (_sz, [_i64] * 6 + [_int]),

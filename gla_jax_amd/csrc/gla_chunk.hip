@@ -15,7 +15,7 @@ struct ChunkPlan {
     size_t prod = 0, decay = 0, states = 0;   // byte sizes, each rounded up to 256
     size_t scale_off = 0;                     // where the products' exponents start inside the decay region
     size_t resid = 0;                         // the forward residual: N + 1 states per (b,h), the last one final
-    // Head dimension 256 runs as two passes of the 128-feature kernels over 2H heads (gla_chunk_split.hip); the
+    // Head dimension 256 runs as two passes of the 128-feature kernels over 2H heads (gla_split.hip); the
     // sizes above are then those of one such pass, and:
     bool split = false;
     size_t rows = 0;                          // one [B,T,H,256] array of the element type
@@ -191,7 +191,7 @@ static int chunk_fwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t
                           key, query, hT_cross, out2, states ? (unsigned char *)states + p.resid : nullptr, ws, sub,
                           p.wide);
         if (e) return e;
-        e = p.wide ? launch_sum_rows(st, B * T * H, out, (const float *)out1, (const float *)out2, 1)
+        e = p.wide ? launch_sum_rows(st, dtype, B * T * H, out, (const float *)out1, (const float *)out2, 1)
                    : launch_add_rows(st, dtype, B * T * H, out, out2, 1);
         if (e) return e;
         return launch_hidden_blocks(st, hidden_dtype, B * H, hidden_final, hT_same, hT_cross, 0);
@@ -315,11 +315,11 @@ static int chunk_bwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t
                           dq2, ws, sub, p.wide);
         if (e) return e;
         if (p.wide) {
-            e = launch_sum_rows(st, rows, dquery, (const float *)dq1, (const float *)dq2, 0);
+            e = launch_sum_rows(st, dtype, rows, dquery, (const float *)dq1, (const float *)dq2, 0);
             if (e) return e;
-            e = launch_sum_rows(st, rows, dkey, (const float *)dk1, (const float *)dk2, 0);
+            e = launch_sum_rows(st, dtype, rows, dkey, (const float *)dk1, (const float *)dk2, 0);
             if (e) return e;
-            e = launch_sum_rows(st, rows, dvalue, (const float *)dv1, (const float *)dv2, 1);
+            e = launch_sum_rows(st, dtype, rows, dvalue, (const float *)dv1, (const float *)dv2, 1);
             if (e) return e;
         } else {
             e = launch_add_rows(st, dtype, rows, dquery, dq2, 0);

@@ -34,7 +34,7 @@
 namespace gla {
 
 // WIDE: dv, dk and dq are float arrays (the sums of two such runs are rounded once: head dimension 256,
-// gla_chunk_split.hip).
+// gla_split.hip).
 template <typename T, int C, int D, int DM, bool WIDE>
 __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k,

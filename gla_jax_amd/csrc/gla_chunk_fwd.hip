@@ -22,7 +22,7 @@ namespace gla {
 // Resources: two tiles (keys of all but the last sub-block, values), 32 staged state rows and a table
 // fit twice into a CU's LDS, and the register budget is held to what lets two workgroups share a CU, so
 // that one loads while the other computes.
-// WIDE: `out` is a float array (the sum of two such runs is rounded once: head dimension 256, gla_chunk_split.hip).
+// WIDE: `out` is a float array (the sum of two such runs is rounded once: head dimension 256, gla_split.hip).
 template <typename T, int C, int D, int DM, bool WIDE>
 __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C / 32))) void chunk_out_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k, const T *__restrict__ q,

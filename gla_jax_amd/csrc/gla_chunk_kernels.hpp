@@ -2,12 +2,13 @@
 #pragma once
 
 #include "gla_common.hpp"
+#include "gla_split.hpp"
 
 namespace gla {
 
 // (T, C, D) combinations that are compiled.  C = tokens per chunk handled by one workgroup
 // (C/16 waves), D = head dimension (DK == DV, gla.py:499).  Head dimension 256 has no kernels of its own: it runs
-// as four problems of head dimension 128 (gla_chunk_split.hip).  D = 32 is the
+// as four problems of head dimension 128 (gla_split.hip).  D = 32 is the
 // smallest head dimension whose feature contractions fill one k-step of the 16x16x32 matrix instruction; head
 // dimension 16 (the smallest the reference's score kernel takes, gla.py:975) runs on those kernels with its
 // rows padded by zeros on the way in.
@@ -54,17 +55,5 @@ template <typename T, int C, int D, int DM, bool WIDE = false>
 int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
                       const void *q, const void *dout, const void *statesN, const void *dstatesT,
                       const void *dstatesN, float *dg, void *dv, void *dk, void *dq);
-
-// ---- head dimension 256 as four problems of head dimension 128 (gla_chunk_split.hip) --------------------------
-// rows = number of 256-element rows; dtype / hdt = gla_dtype of the elements
-// dst[row][j] = src[row][j ^ 128]
-int launch_swap_halves(hipStream_t st, int dtype, int64_t rows, void *dst, const void *src);
-// dst[row][j] += src[row][j], or src[row][j ^ 128] when swapped != 0 (summed in fp32, rounded once)
-int launch_add_rows(hipStream_t st, int dtype, int64_t rows, void *dst, const void *src, int swapped);
-// dst[row][j] = bf16(a[row][j] + b[row][j]), or b[row][j ^ 128] when swapped != 0
-int launch_sum_rows(hipStream_t st, int64_t rows, void *dst, const float *a, const float *b, int swapped);
-// full [BH][256][256] <-> same [BH][2][128][128] (block a = rows and columns of half a) and cross (block a = rows
-// of half a, columns of the other half); gather != 0: full -> blocks, else blocks -> full
-int launch_hidden_blocks(hipStream_t st, int hdt, int64_t BH, void *full, void *same, void *cross, int gather);
 
 }  // namespace gla

@@ -9,6 +9,7 @@
 // operand, does 3*4*R FMAs and its partial sums are reduced over 16 lanes by xor-shuffles.
 #include "gla_common.hpp"
 #include "gla_recurrent_stream.hpp"
+#include "gla_split.hpp"
 
 namespace gla {
 
@@ -422,18 +423,19 @@ template <typename T, typename TO>
 static int launch_bwd(hipStream_t st, int B, int T_len, int H, int DK, int DV, int reverse, int hdt,
                       const void *h0, const float *g, const void *v, const void *k, const void *q,
                       const void * /* hidden_final: recomputed in fp32 by sweep 1 */, const void *dhT,
-                      const void *dout, void *dh0, float *dg, void *dv, void *dk, void *dq)
+                      const void *dout, void *dh0, float *dg, void *dv, void *dk, void *dq, int wide)
 {
     dim3 grid(H, B), block(DK / 16 * 64);
     // bf16 data at head dimensions 64 and 128 runs both sweeps on the matrix cores, whatever the type of dout
     if (sizeof(T) == 2 && (DK == 64 || DK == 128)) {
         const int dout_f32 = sizeof(TO) == 4;
         int e = launch_recurrent_stream_dq(st, B, T_len, H, DK, reverse, hdt, dout_f32, h0, g, v, k, q, dhT, dout, dq,
-                                           dg);
+                                           dg, wide);
         if (e) return e;
         return launch_recurrent_stream_rev(st, B, T_len, H, DK, reverse, hdt, dout_f32, g, v, k, q, dhT, dout, dh0, dg,
-                                           dv, dk);
+                                           dv, dk, wide);
     }
+    if (wide && sizeof(T) != 4) return GLA_ERR_UNSUPPORTED;   // float gradients: the matrix-core kernels or float data
 #define GLA_BWD_CASE(RV_, U_, TB_)                                                                      \
     do {                                                                                                \
         hipLaunchKernelGGL((recurrent_bwd_dq_kernel<T, TO, RV_, U_>), grid, block, 0, st,               \
@@ -471,10 +473,30 @@ static int check_recurrent(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t 
 
 }  // namespace gla
 
-extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                                 gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
-                                 const void *hidden_init, const float *log_fgate, const void *value,
-                                 const void *key, const void *query, void *hidden_final, void *out)
+// ---- head dimension 256 as four problems of head dimension 128 (gla_split.hip) ---------------------------------
+// Two passes of the 128-feature kernels over 2H heads, their results left in fp32 and added with one rounding.
+// rows: one [B,T,H,256] array of floats; hid: one [B,2H,128,128] array of states (sized for fp32 states).
+namespace gla {
+struct SplitSizes {
+    size_t rows_e, rows_f32, hid;
+    SplitSizes(int64_t B, int64_t T, int64_t H, int dtype)
+        : rows_e(round_up256((size_t)B * T * H * 256 * (dtype == GLA_BF16 ? 2 : 4))),
+          rows_f32(round_up256((size_t)B * T * H * 256 * 4)), hid(round_up256((size_t)B * 2 * H * 128 * 128 * 4))
+    {
+    }
+    static size_t round_up256(size_t x) { return (x + 255) & ~(size_t)255; }
+    // forward: value rows with their halves exchanged, both passes' out, hidden_init and hidden_final in blocks
+    size_t fwd() const { return rows_e + 2 * rows_f32 + 4 * hid; }
+    // backward: value and dout rows exchanged, both passes' dq, dk, dv, the second pass's d(log_fgate), hidden_init,
+    // dhidden_final and dhidden_init in blocks
+    size_t bwd() const { return rows_e + rows_f32 + 7 * rows_f32 + 6 * hid; }
+};
+}  // namespace gla
+
+static int recurrent_fwd_run(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, gla_dtype dtype,
+                             gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse, const void *hidden_init,
+                             const float *log_fgate, const void *value, const void *key, const void *query,
+                             void *hidden_final, void *out)
 {
     int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, hidden_dtype, out_dtype);
     if (rc) return rc;
@@ -503,12 +525,76 @@ extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, 
                                          query, hidden_final, out);
 }
 
-extern "C" int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
                                  gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
                                  const void *hidden_init, const float *log_fgate, const void *value,
-                                 const void *key, const void *query, const void *hidden_final,
-                                 const void *dhidden_final, const void *dout, void *dhidden_init,
-                                 float *dlog_fgate, void *dvalue, void *dkey, void *dquery)
+                                 const void *key, const void *query, void *hidden_final, void *out)
+{
+    return recurrent_fwd_run(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init, log_fgate,
+                             value, key, query, hidden_final, out);
+}
+
+extern "C" size_t gla_recurrent_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                                    gla_dtype dtype)
+{
+    if (gla::check_recurrent(B, T, H, DK, DV, dtype, GLA_F32, GLA_F32) || DK != 256 || 2 * H > 65535) return 0;
+    return gla::SplitSizes(B, T, H, dtype).fwd();
+}
+
+extern "C" size_t gla_recurrent_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                                    gla_dtype dtype)
+{
+    if (gla::check_recurrent(B, T, H, DK, DV, dtype, GLA_F32, GLA_F32) || DK != 256 || 2 * H > 65535) return 0;
+    return gla::SplitSizes(B, T, H, dtype).bwd();
+}
+
+extern "C" int gla_recurrent_fwd_ws(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                    gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
+                                    const void *hidden_init, const float *log_fgate, const void *value,
+                                    const void *key, const void *query, void *hidden_final, void *out,
+                                    void *workspace, size_t workspace_bytes)
+{
+    const size_t need = gla_recurrent_fwd_workspace_bytes(B, T, H, DK, DV, dtype);
+    if (!need)      // every other head dimension needs no workspace
+        return recurrent_fwd_run(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
+                                 log_fgate, value, key, query, hidden_final, out);
+    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, hidden_dtype, out_dtype);
+    if (rc) return rc;
+    const void *ptrs[] = {hidden_init, log_fgate, value, key, query, hidden_final, out};
+    for (const void *p : ptrs) {
+        if (!p) return GLA_ERR_NULL;
+        if (!gla::aligned16(p)) return GLA_ERR_ALIGN;
+    }
+    if (!workspace || workspace_bytes < need) return GLA_ERR_WORKSPACE;
+    if (!gla::aligned16(workspace)) return GLA_ERR_ALIGN;
+    const gla::SplitSizes z(B, T, H, dtype);
+    hipStream_t st = (hipStream_t)stream;
+    unsigned char *ws = (unsigned char *)workspace;
+    unsigned char *v_sw = ws, *out1 = v_sw + z.rows_e, *out2 = out1 + z.rows_f32, *h0_same = out2 + z.rows_f32,
+                  *h0_cross = h0_same + z.hid, *hT_same = h0_cross + z.hid, *hT_cross = hT_same + z.hid;
+    int e = gla::launch_hidden_blocks(st, hidden_dtype, B * H, const_cast<void *>(hidden_init), h0_same, h0_cross, 1);
+    if (e) return e;
+    e = gla::launch_swap_halves(st, dtype, B * T * H, v_sw, value);
+    if (e) return e;
+    // key half a with value half a on the arrays as they lie, then key half a with the other value half; `out` of
+    // both in fp32 (the recurrent_gla_naive flavour of the 128-feature kernels)
+    e = recurrent_fwd_run(stream, B, T, 2 * H, 128, 128, dtype, hidden_dtype, GLA_F32, reverse, h0_same, log_fgate,
+                          value, key, query, hT_same, out1);
+    if (e) return e;
+    e = recurrent_fwd_run(stream, B, T, 2 * H, 128, 128, dtype, hidden_dtype, GLA_F32, reverse, h0_cross, log_fgate, v_sw,
+                          key, query, hT_cross, out2);
+    if (e) return e;
+    e = gla::launch_sum_rows(st, out_dtype, B * T * H, out, (const float *)out1, (const float *)out2, 1);
+    if (e) return e;
+    return gla::launch_hidden_blocks(st, hidden_dtype, B * H, hidden_final, hT_same, hT_cross, 0);
+}
+
+// wide != 0: dvalue, dkey, dquery are float arrays whatever `dtype` is
+static int recurrent_bwd_run(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, gla_dtype dtype,
+                             gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse, const void *hidden_init,
+                             const float *log_fgate, const void *value, const void *key, const void *query,
+                             const void *hidden_final, const void *dhidden_final, const void *dout,
+                             void *dhidden_init, float *dlog_fgate, void *dvalue, void *dkey, void *dquery, int wide)
 {
     int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, hidden_dtype, out_dtype);
     if (rc) return rc;
@@ -522,12 +608,82 @@ extern "C" int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, 
     if (dtype == GLA_BF16 && out_dtype == GLA_BF16)
         return gla::launch_bwd<__bf16, __bf16>(st, B, T, H, DK, DV, reverse, hidden_dtype, hidden_init, log_fgate, value,
                                                key, query, hidden_final, dhidden_final, dout, dhidden_init,
-                                               dlog_fgate, dvalue, dkey, dquery);
+                                               dlog_fgate, dvalue, dkey, dquery, wide);
     if (dtype == GLA_BF16)
         return gla::launch_bwd<__bf16, float>(st, B, T, H, DK, DV, reverse, hidden_dtype, hidden_init, log_fgate, value,
                                               key, query, hidden_final, dhidden_final, dout, dhidden_init,
-                                              dlog_fgate, dvalue, dkey, dquery);
+                                              dlog_fgate, dvalue, dkey, dquery, wide);
     return gla::launch_bwd<float, float>(st, B, T, H, DK, DV, reverse, hidden_dtype, hidden_init, log_fgate, value, key,
                                          query, hidden_final, dhidden_final, dout, dhidden_init, dlog_fgate,
-                                         dvalue, dkey, dquery);
+                                         dvalue, dkey, dquery, wide);
+}
+
+extern "C" int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                 gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
+                                 const void *hidden_init, const float *log_fgate, const void *value,
+                                 const void *key, const void *query, const void *hidden_final,
+                                 const void *dhidden_final, const void *dout, void *dhidden_init,
+                                 float *dlog_fgate, void *dvalue, void *dkey, void *dquery)
+{
+    return recurrent_bwd_run(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init, log_fgate,
+                             value, key, query, hidden_final, dhidden_final, dout, dhidden_init, dlog_fgate, dvalue,
+                             dkey, dquery, 0);
+}
+
+extern "C" int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                    gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
+                                    const void *hidden_init, const float *log_fgate, const void *value,
+                                    const void *key, const void *query, const void *hidden_final,
+                                    const void *dhidden_final, const void *dout, void *dhidden_init,
+                                    float *dlog_fgate, void *dvalue, void *dkey, void *dquery, void *workspace,
+                                    size_t workspace_bytes)
+{
+    const size_t need = gla_recurrent_bwd_workspace_bytes(B, T, H, DK, DV, dtype);
+    if (!need)
+        return recurrent_bwd_run(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
+                                 log_fgate, value, key, query, hidden_final, dhidden_final, dout, dhidden_init,
+                                 dlog_fgate, dvalue, dkey, dquery, 0);
+    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, hidden_dtype, out_dtype);
+    if (rc) return rc;
+    const void *ptrs[] = {hidden_init, log_fgate, value, key, query, hidden_final, dhidden_final,
+                          dout, dhidden_init, dlog_fgate, dvalue, dkey, dquery};
+    for (const void *p : ptrs) {
+        if (!p) return GLA_ERR_NULL;
+        if (!gla::aligned16(p)) return GLA_ERR_ALIGN;
+    }
+    if (!workspace || workspace_bytes < need) return GLA_ERR_WORKSPACE;
+    if (!gla::aligned16(workspace)) return GLA_ERR_ALIGN;
+    const gla::SplitSizes z(B, T, H, dtype);
+    hipStream_t st = (hipStream_t)stream;
+    unsigned char *ws = (unsigned char *)workspace;
+    unsigned char *v_sw = ws, *do_sw = v_sw + z.rows_e, *dg2 = do_sw + z.rows_f32, *dq1 = dg2 + z.rows_f32,
+                  *dq2 = dq1 + z.rows_f32, *dk1 = dq2 + z.rows_f32, *dk2 = dk1 + z.rows_f32, *dv1 = dk2 + z.rows_f32,
+                  *dv2 = dv1 + z.rows_f32, *h0_same = dv2 + z.rows_f32, *h0_cross = h0_same + z.hid,
+                  *dhT_same = h0_cross + z.hid, *dhT_cross = dhT_same + z.hid, *dh0_same = dhT_cross + z.hid,
+                  *dh0_cross = dh0_same + z.hid;
+    const int64_t rows = B * T * H;
+    int e = gla::launch_hidden_blocks(st, hidden_dtype, B * H, const_cast<void *>(hidden_init), h0_same, h0_cross, 1);
+    if (e) return e;
+    e = gla::launch_hidden_blocks(st, hidden_dtype, B * H, const_cast<void *>(dhidden_final), dhT_same, dhT_cross, 1);
+    if (e) return e;
+    e = gla::launch_swap_halves(st, dtype, rows, v_sw, value);
+    if (e) return e;
+    e = gla::launch_swap_halves(st, out_dtype, rows, do_sw, dout);
+    if (e) return e;
+    // hidden_final is not read by the kernels (sweep 1 forms the final state again in fp32); it is handed on as it is
+    e = recurrent_bwd_run(stream, B, T, 2 * H, 128, 128, dtype, hidden_dtype, out_dtype, reverse, h0_same, log_fgate,
+                          value, key, query, hidden_final, dhT_same, dout, dh0_same, dlog_fgate, dv1, dk1, dq1, 1);
+    if (e) return e;
+    e = recurrent_bwd_run(stream, B, T, 2 * H, 128, 128, dtype, hidden_dtype, out_dtype, reverse, h0_cross, log_fgate,
+                          v_sw, key, query, hidden_final, dhT_cross, do_sw, dh0_cross, (float *)dg2, dv2, dk2, dq2, 1);
+    if (e) return e;
+    e = gla::launch_sum_rows(st, dtype, rows, dquery, (const float *)dq1, (const float *)dq2, 0);
+    if (e) return e;
+    e = gla::launch_sum_rows(st, dtype, rows, dkey, (const float *)dk1, (const float *)dk2, 0);
+    if (e) return e;
+    e = gla::launch_sum_rows(st, dtype, rows, dvalue, (const float *)dv1, (const float *)dv2, 1);
+    if (e) return e;
+    e = gla::launch_add_rows(st, GLA_F32, rows, dlog_fgate, dg2, 0);
+    if (e) return e;
+    return gla::launch_hidden_blocks(st, hidden_dtype, B * H, dhidden_init, dh0_same, dh0_cross, 0);
 }

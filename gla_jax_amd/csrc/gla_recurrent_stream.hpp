@@ -13,20 +13,22 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
                                 void *hT, void *out);
 
 // Sweep 1 of the backward: dq, and q*dq in fp32 into `qdq` (the last step's carries sum_v dhT * (final state)
-// on top).  dout_f32 != 0: `dout` is float (the recurrent_gla_naive flavour), else bf16.
+// on top).  dout_f32 != 0: `dout` is float (the recurrent_gla_naive flavour), else bf16.  wide != 0 (head dimension
+// 128 only): `dq` is a float array, for the two passes that make up head dimension 256.
 int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
                                const void *h0, const float *g, const void *v, const void *k, const void *q,
-                               const void *dhT, const void *dout, void *dq, float *qdq);
+                               const void *dhT, const void *dout, void *dq, float *qdq, int wide = 0);
 
 // The same sweep with two waves per sub-block (head dimension 64).
 int launch_recurrent_stream_dq2(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
                                 const void *h0, const float *g, const void *v, const void *k, const void *q,
                                 const void *dhT, const void *dout, void *dq, float *qdq);
 
-// Sweep 2: dk, dv, dh0 and dlog_fgate (`dg` holds sweep 1's q*dq on entry).
+// Sweep 2: dk, dv, dh0 and dlog_fgate (`dg` holds sweep 1's q*dq on entry).  wide != 0 (head dimension 128 only):
+// `dv` and `dk` are float arrays.
 int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
                                 const float *g, const void *v, const void *k, const void *q, const void *dhT,
-                                const void *dout, void *dh0, float *dg, void *dv, void *dk);
+                                const void *dout, void *dh0, float *dg, void *dv, void *dk, int wide = 0);
 
 // The same sweep with two waves per sub-block (head dimension 64).
 int launch_recurrent_stream_rev2(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,

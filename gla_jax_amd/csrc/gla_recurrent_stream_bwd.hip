@@ -24,13 +24,16 @@ typedef __bf16 BT;
 // ---------------------------------------------------------------------------------------------------
 // sweep 1
 // ---------------------------------------------------------------------------------------------------
-template <typename TO, int C, int D>
+// WIDE: dq is a float array (head dimension 256 adds two such runs and rounds once, gla_split.hip)
+template <typename TO, int C, int D, bool WIDE>
 __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
     const void *__restrict__ h0, const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k,
-    const BT *__restrict__ q, const void *__restrict__ dhT, const TO *__restrict__ dout, BT *__restrict__ dq,
-    float *__restrict__ qdq, int T_len, int H, int reverse, int hdt)
+    const BT *__restrict__ q, const void *__restrict__ dhT, const TO *__restrict__ dout,
+    std::conditional_t<WIDE, float, BT> *__restrict__ dq, float *__restrict__ qdq, int T_len, int H, int reverse,
+    int hdt)
 {
     typedef BT T;
+    typedef std::conditional_t<WIDE, float, BT> TG;
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16, RT = NT / NB;
     static_assert(NT % NB == 0, "every wave owns the same number of state row tiles");
     constexpr int LS = TileGeom<T, D>::kStride;
@@ -288,7 +291,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
                 prod.v[e] = a[e] * o[e];
             }
             if (valid) {
-                st8(dq + row + fo + 8 * c, pack8<T>(o));
+                st8(dq + row + fo + 8 * c, pack8<TG>(o));
                 st8(qdq + row + fo + 8 * c, prod);
             }
         }
@@ -355,13 +358,16 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_dq_kernel(
 //   dS_in = diag(e^{Lend}) dS' + sum_i (q e^{L})_i do_i^T     (a Horner chain over the sub-blocks, last first)
 // dS' is the gradient w.r.t. the state after the block.
 // ---------------------------------------------------------------------------------------------------
-template <typename TO, int C, int D>
+// WIDE: dv and dk are float arrays (see sweep 1)
+template <typename TO, int C, int D, bool WIDE>
 __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
     const float *__restrict__ g, const BT *__restrict__ v, const BT *__restrict__ k, const BT *__restrict__ q,
     const void *__restrict__ dhT, const TO *__restrict__ dout, void *__restrict__ dh0,
-    float *__restrict__ dg, BT *__restrict__ dv, BT *__restrict__ dk, int T_len, int H, int reverse, int hdt)
+    float *__restrict__ dg, std::conditional_t<WIDE, float, BT> *__restrict__ dv,
+    std::conditional_t<WIDE, float, BT> *__restrict__ dk, int T_len, int H, int reverse, int hdt)
 {
     typedef BT T;
+    typedef std::conditional_t<WIDE, float, BT> TG;
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16, RT = NT / NB;
     static_assert(NT % NB == 0, "every wave owns the same number of state row tiles");
     constexpr int LS = TileGeom<T, D>::kStride;
@@ -681,7 +687,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                 float o[8];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
-                if (valid) st8(dv + row + fo + 8 * c, pack8<T>(o));
+                if (valid) st8(dv + row + fo + 8 * c, pack8<TG>(o));
             }
             // -- dk slice: dS' v first, then the later sub-blocks in descending order
             {
@@ -725,7 +731,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                     sfx.v[e] = suffix_sum_rows(qdq[8 * ks + e] - kk[e] * o[e]);
                     qdq[8 * ks + e] = sfx.v[e];
                 }
-                if (valid) st8(dk + row + fo + 8 * c, pack8<T>(o));
+                if (valid) st8(dk + row + fo + 8 * c, pack8<TG>(o));
                 if (r == 0) st8(dltab + w * D + fo + 8 * c, sfx);
             }
         }
@@ -784,7 +790,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_rev_kernel(
                 store_hidden1(dh0, hdt, bh * D * D + (int64_t)(16 * (w + i * NB) + 4 * c + e) * D + 16 * nt + r, DS[i][nt][e]);
 }
 
-template <typename TO, int C, int D>
+template <typename TO, int C, int D, bool WIDE>
 static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, int hdt, const void *h0, const float *g,
                      const void *v, const void *k, const void *q, const void *dhT, const void *dout, void *dq,
                      float *qdq)
@@ -794,16 +800,16 @@ static int launch_dq(hipStream_t st, int B, int T_len, int H, int reverse, int h
     constexpr int XS = 32 + 16 / (int)sizeof(T);
     const size_t lds = ((size_t)(3 * C + 2 * D) * LS + (size_t)(C / 16) * 2 * 16 * XS) * sizeof(T) +
                        (size_t)(C / 16) * D * sizeof(float);
-    auto kern = recurrent_stream_dq_kernel<TO, C, D>;
+    auto kern = recurrent_stream_dq_kernel<TO, C, D, WIDE>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, h0, g, (const T *)v, (const T *)k, (const T *)q,
-                       dhT, (const TO *)dout, (T *)dq, qdq, T_len, H, reverse, hdt);
+                       dhT, (const TO *)dout, (std::conditional_t<WIDE, float, T> *)dq, qdq, T_len, H, reverse, hdt);
     return launch_status();
 }
 
-template <typename TO, int C, int D>
+template <typename TO, int C, int D, bool WIDE>
 static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, int hdt, const float *g, const void *v,
                       const void *k, const void *q, const void *dhT, const void *dout, void *dh0,
                       float *dg, void *dv, void *dk)
@@ -814,39 +820,46 @@ static int launch_rev(hipStream_t st, int B, int T_len, int H, int reverse, int 
     const size_t lds = ((size_t)(3 * C + 2 * D + (sizeof(TO) == 4 ? C : 0)) * LS + (size_t)(C / 16) * 2 * 16 * XS) *
                            sizeof(T) +
                        (size_t)(2 * (C / 16) + 2) * D * sizeof(float);
-    auto kern = recurrent_stream_rev_kernel<TO, C, D>;
+    auto kern = recurrent_stream_rev_kernel<TO, C, D, WIDE>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
-                       dhT, (const TO *)dout, dh0, dg, (T *)dv, (T *)dk, T_len, H, reverse, hdt);
+                       dhT, (const TO *)dout, dh0, dg, (std::conditional_t<WIDE, float, T> *)dv,
+                       (std::conditional_t<WIDE, float, T> *)dk, T_len, H, reverse, hdt);
     return launch_status();
 }
 
 int launch_recurrent_stream_rev(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
                                 const float *g, const void *v, const void *k, const void *q, const void *dhT,
-                                const void *dout, void *dh0, float *dg, void *dv, void *dk)
+                                const void *dout, void *dh0, float *dg, void *dv, void *dk, int wide)
 {
-    if (D == 64)
+    if (D == 64 && !wide)
         return launch_recurrent_stream_rev2(st, B, T_len, H, D, reverse, hdt, dout_f32, g, v, k, q, dhT, dout, dh0, dg,
                                             dv, dk);
-    if (D == 128 && dout_f32)
-        return launch_rev<float, 64, 128>(st, B, T_len, H, reverse, hdt, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
-    if (D == 128) return launch_rev<BT, 64, 128>(st, B, T_len, H, reverse, hdt, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
-    return GLA_ERR_UNSUPPORTED;
+    if (D != 128) return GLA_ERR_UNSUPPORTED;
+    if (wide)
+        return dout_f32
+                   ? launch_rev<float, 64, 128, true>(st, B, T_len, H, reverse, hdt, g, v, k, q, dhT, dout, dh0, dg, dv, dk)
+                   : launch_rev<BT, 64, 128, true>(st, B, T_len, H, reverse, hdt, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
+    return dout_f32 ? launch_rev<float, 64, 128, false>(st, B, T_len, H, reverse, hdt, g, v, k, q, dhT, dout, dh0, dg, dv, dk)
+                    : launch_rev<BT, 64, 128, false>(st, B, T_len, H, reverse, hdt, g, v, k, q, dhT, dout, dh0, dg, dv, dk);
 }
 
 int launch_recurrent_stream_dq(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, int dout_f32,
                                const void *h0, const float *g, const void *v, const void *k, const void *q,
-                               const void *dhT, const void *dout, void *dq, float *qdq)
+                               const void *dhT, const void *dout, void *dq, float *qdq, int wide)
 {
-    if (D == 64)
+    if (D == 64 && !wide)
         return launch_recurrent_stream_dq2(st, B, T_len, H, D, reverse, hdt, dout_f32, h0, g, v, k, q, dhT, dout, dq,
                                            qdq);
-    if (D == 128 && dout_f32)
-        return launch_dq<float, 64, 128>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, dhT, dout, dq, qdq);
-    if (D == 128) return launch_dq<BT, 64, 128>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, dhT, dout, dq, qdq);
-    return GLA_ERR_UNSUPPORTED;
+    if (D != 128) return GLA_ERR_UNSUPPORTED;
+    if (wide)
+        return dout_f32
+                   ? launch_dq<float, 64, 128, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, dhT, dout, dq, qdq)
+                   : launch_dq<BT, 64, 128, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, dhT, dout, dq, qdq);
+    return dout_f32 ? launch_dq<float, 64, 128, false>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, dhT, dout, dq, qdq)
+                    : launch_dq<BT, 64, 128, false>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, dhT, dout, dq, qdq);
 }
 
 }  // namespace gla

@@ -1,4 +1,4 @@
-// chunk_gla at head dimension 256 as four problems of head dimension 128.
+// chunk_gla and recurrent_gla at head dimension 256 as four problems of head dimension 128.
 //
 // The recurrence is a sum over key features and independent over value features: with the key features split
 // into halves a and the value features into halves b,
@@ -10,7 +10,7 @@
 // holds the small kernels around those runs: exchanging halves, adding the two runs' results (for bf16 data both runs
 // leave out, dq, dk and dv in fp32 and the sum is rounded once, as one kernel over all 256 features would round it),
 // and cutting the [256,256] states into their four [128,128] blocks and back.
-#include "gla_chunk_kernels.hpp"
+#include "gla_split.hpp"
 
 namespace gla {
 
@@ -120,11 +120,14 @@ int launch_add_rows(hipStream_t st, int dtype, int64_t rows, void *dst, const vo
     return launch_status();
 }
 
-int launch_sum_rows(hipStream_t st, int64_t rows, void *dst, const float *a, const float *b, int swapped)
+int launch_sum_rows(hipStream_t st, int dtype, int64_t rows, void *dst, const float *a, const float *b, int swapped)
 {
     const int64_t n8 = rows * kRow / 8;
     if (n8 > 0x7fffffffLL * 256) return GLA_ERR_SHAPE;
-    hipLaunchKernelGGL(sum_rows_kernel<__bf16>, grid_for(n8), dim3(256), 0, st, (__bf16 *)dst, a, b, n8, swapped);
+    if (dtype == GLA_BF16)
+        hipLaunchKernelGGL(sum_rows_kernel<__bf16>, grid_for(n8), dim3(256), 0, st, (__bf16 *)dst, a, b, n8, swapped);
+    else
+        hipLaunchKernelGGL(sum_rows_kernel<float>, grid_for(n8), dim3(256), 0, st, (float *)dst, a, b, n8, swapped);
     return launch_status();
 }
 

@@ -271,9 +271,13 @@ class _RecurrentGLA(torch.autograd.Function):
         odt = _lib.GLA_F32 if out_fp32 else dt
         hT = torch.empty_like(h0)
         out = torch.empty(v.shape, dtype=torch.float32 if out_fp32 else v.dtype, device=v.device)
-        rc = lib.gla_recurrent_fwd(_stream(), B, T, H, DK, DV, dt, _DT[h0.dtype], odt, int(bool(reverse)), _ptr(h0),
-                                   _ptr(g), _ptr(v), _ptr(k), _ptr(q), _ptr(hT), _ptr(out))
-        _lib.check("gla_recurrent_fwd", rc)
+        # a workspace is needed at head dimension 256 only (two passes of the 128-feature kernels)
+        ws_bytes = lib.gla_recurrent_fwd_workspace_bytes(B, T, H, DK, DV, dt)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=v.device) if ws_bytes else None
+        rc = lib.gla_recurrent_fwd_ws(_stream(), B, T, H, DK, DV, dt, _DT[h0.dtype], odt, int(bool(reverse)), _ptr(h0),
+                                      _ptr(g), _ptr(v), _ptr(k), _ptr(q), _ptr(hT), _ptr(out),
+                                      _ptr(ws) if ws_bytes else None, ws_bytes)
+        _lib.check("gla_recurrent_fwd_ws", rc)
         return hT, out
 
     @staticmethod
@@ -314,11 +318,13 @@ class _RecurrentGLABwd(torch.autograd.Function):
         dh0 = torch.empty_like(h0)
         dg = torch.empty_like(g)
         dv, dk, dq = torch.empty_like(v), torch.empty_like(k), torch.empty_like(q)
-        rc = lib.gla_recurrent_bwd(_stream(), B, T, H, DK, DV, dt, _DT[h0.dtype], odt, int(bool(reverse)), _ptr(h0),
-                                   _ptr(g),
-                                   _ptr(v), _ptr(k), _ptr(q), _ptr(hTc), _ptr(dhT), _ptr(dout),
-                                   _ptr(dh0), _ptr(dg), _ptr(dv), _ptr(dk), _ptr(dq))
-        _lib.check("gla_recurrent_bwd", rc)
+        ws_bytes = lib.gla_recurrent_bwd_workspace_bytes(B, T, H, DK, DV, dt)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=v.device) if ws_bytes else None
+        rc = lib.gla_recurrent_bwd_ws(_stream(), B, T, H, DK, DV, dt, _DT[h0.dtype], odt, int(bool(reverse)), _ptr(h0),
+                                      _ptr(g), _ptr(v), _ptr(k), _ptr(q), _ptr(hTc), _ptr(dhT), _ptr(dout),
+                                      _ptr(dh0), _ptr(dg), _ptr(dv), _ptr(dk), _ptr(dq),
+                                      _ptr(ws) if ws_bytes else None, ws_bytes)
+        _lib.check("gla_recurrent_bwd_ws", rc)
         return dh0, dg, dv, dk, dq
 
     @staticmethod

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define GLA_HIP_ABI_VERSION 2
+#define GLA_HIP_ABI_VERSION 3
 
 typedef enum gla_dtype {
     GLA_F32 = 0,
@@ -108,6 +108,28 @@ int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK,
                       const void *key, const void *query, const void *hidden_final,
                       const void *dhidden_final, const void *dout,
                       void *dhidden_init, float *dlog_fgate, void *dvalue, void *dkey, void *dquery);
+
+/* The same two rules (gla.py:99-170, 172-269) with a caller-provided workspace.  At head dimension 256 the
+ * recurrence then runs as four problems of head dimension 128 (it is a sum over key features and independent over
+ * value features): two passes of the 128-feature kernels over 2H heads, on the matrix cores for bf16 data, with
+ * the passes' results kept in fp32 in the workspace and rounded once.  Without a workspace (the two entry points
+ * above) head dimension 256 runs on per-timestep vector kernels, an order of magnitude slower.  The size
+ * functions return 0 where no workspace is needed; the entry points then ignore `workspace` (NULL is fine) and
+ * behave exactly like the ones above.  Same results within the tolerance either way. */
+size_t gla_recurrent_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, gla_dtype dtype);
+size_t gla_recurrent_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, gla_dtype dtype);
+int gla_recurrent_fwd_ws(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                         gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
+                         const void *hidden_init, const float *log_fgate, const void *value,
+                         const void *key, const void *query,
+                         void *hidden_final, void *out, void *workspace, size_t workspace_bytes);
+int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                         gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
+                         const void *hidden_init, const float *log_fgate, const void *value,
+                         const void *key, const void *query, const void *hidden_final,
+                         const void *dhidden_final, const void *dout,
+                         void *dhidden_init, float *dlog_fgate, void *dvalue, void *dkey, void *dquery,
+                         void *workspace, size_t workspace_bytes);
 
 /* ---- chunk_gla (gla.py:657-692) -------------------------------------------------------------- */
 

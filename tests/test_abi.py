@@ -85,6 +85,15 @@ def test_chunk_plan_and_sizes():
     assert sub + 16 * rows + hid <= lib.gla_chunk_bwd_workspace_bytes(B, T, H, 256, 256, 128, _lib.GLA_BF16) <= (
         sub + 16 * rows + hid + 12 * 256)
     assert lib.gla_chunk_states_bytes(B, T, H, 512, 512, 128, _lib.GLA_BF16) == 0
+    # recurrent_gla: a workspace at head dimension 256 only (both passes' results in fp32 and the exchanged rows)
+    for D in (16, 32, 64, 128):
+        assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, D, D, _lib.GLA_BF16) == 0
+        assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, D, D, _lib.GLA_F32) == 0
+    rows32 = B * T * H * 256 * 4
+    assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, 256, 256, _lib.GLA_BF16) >= rows32 // 2 + 2 * rows32
+    assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, 256, 256, _lib.GLA_BF16) >= rows32 // 2 + 8 * rows32
+    assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, 256, 256, _lib.GLA_F32) >= 9 * rows32
+    assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, 256, 128, _lib.GLA_BF16) == 0      # DK != DV: unsupported
 
 
 def test_entry_points_reject_bad_arguments_without_touching_the_gpu():
@@ -104,6 +113,15 @@ def test_entry_points_reject_bad_arguments_without_touching_the_gpu():
     assert lib.gla_rnn_scan_f32(None, a, a + 4, None, None, None, a, 1, 4, 4, 8, 0) == -6      # 16-byte rows
     # misaligned
     assert lib.gla_recurrent_fwd(None, 1, 8, 1, 64, 64, 1, 1, 1, 0, a + 2, a, a, a, a, a, a) == -6
+    # the workspace variants: ignored where none is needed, checked at head dimension 256
+    rec = lambda D, ws, n: lib.gla_recurrent_fwd_ws(None, 1, 8, 1, D, D, 1, 1, 1, 0, a, a, a, a, a, a, a, ws, n)
+    assert rec(48, None, 0) == -2
+    assert rec(256, None, 0) == -5
+    assert rec(256, a, 64) == -5
+    assert lib.gla_recurrent_bwd_ws(None, 1, 8, 1, 256, 256, 1, 1, 1, 0, a, a, a, a, a, a, a, a, a, a, a, a, a,
+                                    a, 64) == -5
+    assert lib.gla_recurrent_bwd_ws(None, 1, 8, 1, 256, 256, 1, 1, 1, 0, a, a, a, a, a, a, a, a, a, a, a, a, None,
+                                    a, 1 << 40) == -1
     # chunk: not a power of two / not dividing T / unsupported head dim / missing workspace
     args = lambda T, D, C, hd=0: (None, 1, T, 1, D, D, C, 1, hd, a, a, a, a, a, a, a, a)
     assert lib.gla_chunk_fwd(*args(256, 64, 48), a, 1 << 30) == -4

@@ -44,7 +44,7 @@ the case is listed.
 The third is case 43 of the suite's own sweep (tests/test_gpu_sweep.py, which runs it as a known open case), a
 head-dimension-256 case with three resets to -25 in one 64-token chunk.  It passed (0.88 x) while head dimension
 256 had kernels of its own on 32-token tiles and is at 1.63 x in d(log_fgate) since it runs as four problems of head
-dimension 128 (gla_chunk_split.hip): the error is one pair term, rows 11 and 17 of a key feature whose gate
+dimension 128 (gla_split.hip): the error is one pair term, rows 11 and 17 of a key feature whose gate
 gradient is nine RMS large (657 where the RMS is 76), off by 0.5 % where the emulated reference is off by 0.26 %.
 dA = dO V^T of that pair is now the sum of two halves over the value features, each rounded to bf16 on its own; on
 average that costs nothing (40 random head-dimension-256 cases: median 0.90, largest 1.21, against 0.90 and 1.17

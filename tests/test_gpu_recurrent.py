@@ -73,7 +73,7 @@ def test_recurrent_matrix_core_path_over_gate_regimes(T, reverse, D):
     print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads)))
 
 
-@pytest.mark.parametrize("T,D", [(50, 64), (300, 64), (150, 128), (40, 32)])
+@pytest.mark.parametrize("T,D", [(50, 64), (300, 64), (150, 128), (40, 32), (90, 256)])
 def test_recurrent_gla_naive_returns_fp32_out(T, D):
     """The naive flavour (gla.py:26-47): fp32 `out` (promotion at gla.py:37) to fp32 accuracy although the inputs
     are bf16, and an fp32 cotangent for it in the backward.  D=64 and 128 run on the matrix-core kernels (the
