@@ -35,6 +35,10 @@ for _fn in ("gla_chunk_states_bytes", "gla_chunk_fwd_workspace_bytes", "gla_chun
     getattr(_HIP, _fn).restype = ctypes.c_size_t
     getattr(_HIP, _fn).argtypes = [ctypes.c_int64] * 6 + [ctypes.c_int]
 
+for _fn in ("gla_recurrent_fwd_workspace_bytes", "gla_recurrent_bwd_workspace_bytes"):
+    getattr(_HIP, _fn).restype = ctypes.c_size_t
+    getattr(_HIP, _fn).argtypes = [ctypes.c_int64] * 5 + [ctypes.c_int]
+
 _GLA_F32, _GLA_BF16 = 0, 1
 
 
@@ -123,11 +127,22 @@ def recurrent_gla_forward_backward(hidden_init, log_fgate, value, key, query, re
     return _rec_fwd(hidden_init, log_fgate, value, key, query, reverse, out_fp32)[0]
 
 
+def _rec_workspace(key, value, which):
+    """The workspace of a recurrent_gla call as a byte array (head dimension 256 needs one, elsewhere 16 bytes)."""
+    *lead, T, H, DK = key.shape
+    B = 1
+    for s in lead:
+        B *= s
+    n = getattr(_HIP, f"gla_recurrent_{which}_workspace_bytes")(B, T, H, DK, value.shape[-1], _dt(value.dtype))
+    return jax.ShapeDtypeStruct((max(int(n), 16),), jnp.uint8)
+
+
 def _rec_fwd(hidden_init, log_fgate, value, key, query, reverse, out_fp32):
     h0 = _state(hidden_init)
     g = log_fgate.astype(jnp.float32)
-    hT, out = jax.ffi.ffi_call(
-        "GlaRecurrentFwd", (_like(h0), _like(value, jnp.float32 if out_fp32 else None)),
+    hT, out, _ws = jax.ffi.ffi_call(
+        "GlaRecurrentFwd", (_like(h0), _like(value, jnp.float32 if out_fp32 else None),
+                            _rec_workspace(key, value, "fwd")),
         vmap_method="broadcast_all")(h0, g, value, key, query, reverse=bool(reverse))
     res = (h0, g, value, key, query, hT, hidden_init.dtype, log_fgate.dtype)                     # gla.py:169
     return (hT.astype(hidden_init.dtype), out), res
@@ -136,8 +151,9 @@ def _rec_fwd(hidden_init, log_fgate, value, key, query, reverse, out_fp32):
 def _rec_bwd(reverse, out_fp32, res, cotangents):
     h0, g, value, key, query, hT, h_dtype, g_dtype = res
     dhT, dout = cotangents
-    dh0, dg, dv, dk, dq = jax.ffi.ffi_call(
-        "GlaRecurrentBwd", (_like(h0), _like(g), _like(value), _like(key), _like(query)),
+    dh0, dg, dv, dk, dq, _ws = jax.ffi.ffi_call(
+        "GlaRecurrentBwd", (_like(h0), _like(g), _like(value), _like(key), _like(query),
+                            _rec_workspace(key, value, "bwd")),
         vmap_method="broadcast_all")(h0, g, value, key, query, hT, dhT.astype(h0.dtype),
                                      dout.astype(jnp.float32 if out_fp32 else value.dtype),
                                      reverse=bool(reverse))

@@ -107,20 +107,23 @@ ffi::Error ChunkBwd(hipStream_t stream, int64_t chunk_size, ffi::Buffer<ffi::F32
 
 // ---- recurrent_gla -----------------------------------------------------------------------------------------
 // forward rule, recurrent_gla_forward (gla.py:99-170); `reverse` as in gla.py:421-438.  The element type of
-// `out` selects the flavour: the value dtype for recurrent_gla, F32 for recurrent_gla_naive (gla.py:37).
+// `out` selects the flavour: the value dtype for recurrent_gla, F32 for recurrent_gla_naive (gla.py:37).  The last
+// result is a workspace XLA allocates for the call, sized by gla_recurrent_fwd_workspace_bytes on the Python side
+// (head dimension 256 needs one; elsewhere it is a few bytes that nobody reads).
 ffi::Error RecurrentFwd(hipStream_t stream, bool reverse, ffi::AnyBuffer h0, ffi::Buffer<ffi::F32> g,
                         ffi::AnyBuffer v, ffi::AnyBuffer k, ffi::AnyBuffer q, ffi::Result<ffi::AnyBuffer> hT,
-                        ffi::Result<ffi::AnyBuffer> out)
+                        ffi::Result<ffi::AnyBuffer> out, ffi::Result<ffi::AnyBuffer> workspace)
 {
     Dims d = dims_of(k, v);
     gla_dtype dt, hdt, odt;
     if (!d.ok || !dtype_of(v.element_type(), &dt) || !dtype_of(out->element_type(), &odt) ||
         !dtype_of(h0.element_type(), &hdt) || hT->element_type() != h0.element_type())
         return ffi::Error::InvalidArgument("gla_recurrent_fwd: bad operands");
-    return status("gla_recurrent_fwd",
-                  gla_recurrent_fwd(stream, d.B, d.T, d.H, d.DK, d.DV, dt, hdt, odt, reverse ? 1 : 0,
-                                    h0.untyped_data(), g.typed_data(), v.untyped_data(), k.untyped_data(),
-                                    q.untyped_data(), hT->untyped_data(), out->untyped_data()));
+    return status("gla_recurrent_fwd_ws",
+                  gla_recurrent_fwd_ws(stream, d.B, d.T, d.H, d.DK, d.DV, dt, hdt, odt, reverse ? 1 : 0,
+                                       h0.untyped_data(), g.typed_data(), v.untyped_data(), k.untyped_data(),
+                                       q.untyped_data(), hT->untyped_data(), out->untyped_data(),
+                                       workspace->untyped_data(), workspace->size_bytes()));
 }
 
 // backward rule, recurrent_gla_backward (gla.py:172-269); residuals (h0, g, v, k, q, hidden_final), gla.py:169.
@@ -128,7 +131,8 @@ ffi::Error RecurrentBwd(hipStream_t stream, bool reverse, ffi::AnyBuffer h0, ffi
                         ffi::AnyBuffer v, ffi::AnyBuffer k, ffi::AnyBuffer q, ffi::AnyBuffer hT,
                         ffi::AnyBuffer dhT, ffi::AnyBuffer dout, ffi::Result<ffi::AnyBuffer> dh0,
                         ffi::Result<ffi::Buffer<ffi::F32>> dg, ffi::Result<ffi::AnyBuffer> dv,
-                        ffi::Result<ffi::AnyBuffer> dk, ffi::Result<ffi::AnyBuffer> dq)
+                        ffi::Result<ffi::AnyBuffer> dk, ffi::Result<ffi::AnyBuffer> dq,
+                        ffi::Result<ffi::AnyBuffer> workspace)
 {
     Dims d = dims_of(k, v);
     gla_dtype dt, hdt, odt;
@@ -136,12 +140,13 @@ ffi::Error RecurrentBwd(hipStream_t stream, bool reverse, ffi::AnyBuffer h0, ffi
         !dtype_of(h0.element_type(), &hdt) || hT.element_type() != h0.element_type() ||
         dhT.element_type() != h0.element_type() || dh0->element_type() != h0.element_type())
         return ffi::Error::InvalidArgument("gla_recurrent_bwd: bad operands");
-    return status("gla_recurrent_bwd",
-                  gla_recurrent_bwd(stream, d.B, d.T, d.H, d.DK, d.DV, dt, hdt, odt, reverse ? 1 : 0,
-                                    h0.untyped_data(), g.typed_data(), v.untyped_data(), k.untyped_data(),
-                                    q.untyped_data(), hT.untyped_data(), dhT.untyped_data(), dout.untyped_data(),
-                                    dh0->untyped_data(), dg->typed_data(), dv->untyped_data(),
-                                    dk->untyped_data(), dq->untyped_data()));
+    return status("gla_recurrent_bwd_ws",
+                  gla_recurrent_bwd_ws(stream, d.B, d.T, d.H, d.DK, d.DV, dt, hdt, odt, reverse ? 1 : 0,
+                                       h0.untyped_data(), g.typed_data(), v.untyped_data(), k.untyped_data(),
+                                       q.untyped_data(), hT.untyped_data(), dhT.untyped_data(), dout.untyped_data(),
+                                       dh0->untyped_data(), dg->typed_data(), dv->untyped_data(),
+                                       dk->untyped_data(), dq->untyped_data(), workspace->untyped_data(),
+                                       workspace->size_bytes()));
 }
 
 // ---- the scans of ops.py -----------------------------------------------------------------------------------
@@ -223,7 +228,8 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(GlaRecurrentFwd, RecurrentFwd,
                                   .Arg<ffi::AnyBuffer>()
                                   .Arg<ffi::AnyBuffer>()
                                   .Ret<ffi::AnyBuffer>()
-                                  .Ret<ffi::AnyBuffer>());
+                                  .Ret<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>());        // workspace
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(GlaRecurrentBwd, RecurrentBwd,
                               ffi::Ffi::Bind()
@@ -241,7 +247,8 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(GlaRecurrentBwd, RecurrentBwd,
                                   .Ret<ffi::Buffer<ffi::F32>>()
                                   .Ret<ffi::AnyBuffer>()
                                   .Ret<ffi::AnyBuffer>()
-                                  .Ret<ffi::AnyBuffer>());
+                                  .Ret<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>());        // workspace
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(GlaCumsum, Cumsum,
                               ffi::Ffi::Bind()

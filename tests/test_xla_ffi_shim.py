@@ -53,7 +53,7 @@ def test_handlers_call_the_c_abi_as_declared():
     text = _strip_comments(open(CC).read())
     calls = [(m.group(1), _call_args(text, m.end() - 1)) for m in re.finditer(r"\b(gla_[a-z0-9_]+)\s*\(", text)]
     used = {n for n, _ in calls}
-    assert {"gla_chunk_fwd", "gla_chunk_bwd", "gla_recurrent_fwd", "gla_recurrent_bwd", "gla_cumsum_f32",
+    assert {"gla_chunk_fwd", "gla_chunk_bwd", "gla_recurrent_fwd_ws", "gla_recurrent_bwd_ws", "gla_cumsum_f32",
             "gla_rnn_scan_f32", "gla_status_string"} <= used
     for name, nargs in calls:
         assert name in decl, f"{name} is not declared in include/gla_hip.h"
