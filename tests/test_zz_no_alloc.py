@@ -45,6 +45,7 @@ def test_static_entry_point_matches_the_workspace_one():
     _run_pair(lib, _lib, 1, 128, 2, 64, 64, seed=22)             # a smaller input right after: stale contents around it
     _run_pair(lib, _lib, 2, 96, 1, 64, 32, seed=23, dtype=torch.float32)
     _run_pair(lib, _lib, 4, 4096, 6, 128, 128, seed=24)          # the headline shape: 49.1 of the 80 MiB
+    _run_pair(lib, _lib, 1, 256, 2, 256, 128, seed=25)           # head dimension 256: two passes inside the same array
 
 
 def test_static_entry_point_rejects_what_does_not_fit():
