@@ -19,13 +19,13 @@ def _bind(name):
 
 
 @pytest.mark.parametrize("name", ["recurrent_gla", "recurrent_gla_naive"])
-@pytest.mark.parametrize("D", [64, 32])
+@pytest.mark.parametrize("D", [64, 32, 256])
 def test_fp32_state_beside_bf16_arrays_is_not_rounded(name, D):
     """A float32 hidden_init whose values bf16 does NOT hold, beside bf16 value/key/query: the recurrent paths
     load it into their fp32 state as it is and store hidden_final in float32 (gla.py:44-46, 89-97), so the
     final state and the gradient of the initial one match the fp64 oracle to float32 accuracy (1e-4 RMS), far
     below the 2^-9 a cast of the state to bf16 would leave.  D=64 runs on the matrix-core kernels, D=32 on the
-    vector kernels."""
+    vector kernels, D=256 as two passes of the 128-feature matrix-core kernels with the states cut into blocks."""
     fn = _bind(name)
     dtype = torch.bfloat16
     (h0, g, v, k, q), dev = gpu_inputs(2, 200, 2, D, 4.0, seed=21, dtype=dtype)
@@ -48,13 +48,15 @@ def test_fp32_state_beside_bf16_arrays_is_not_rounded(name, D):
     assert err_over_rms(to_np(hT16), exact[5]) > 1e-3
 
 
-def test_chunk_fp32_state_beside_bf16_arrays_enters_the_scan_unrounded():
+@pytest.mark.parametrize("D", [64, 256])
+def test_chunk_fp32_state_beside_bf16_arrays_enters_the_scan_unrounded(D):
     """chunk_gla hands hidden_init to the chunk scan uncast (gla.py:711-716): with keys of zero the final state
     is exactly hidden_init times the total decay, and a float32 hidden_init that bf16 does not hold must come
-    back to float32 accuracy.  Only the copy used as the first chunk's incoming state is rounded (gla.py:720)."""
+    back to float32 accuracy.  Only the copy used as the first chunk's incoming state is rounded (gla.py:720).
+    Head dimension 256 cuts the states into four blocks on the way in and puts them together on the way out."""
     from gla_jax_amd import chunk_gla
     dtype = torch.bfloat16
-    (h0, g, v, k, q), dev = gpu_inputs(2, 256, 2, 64, 4.0, seed=22, dtype=dtype)
+    (h0, g, v, k, q), dev = gpu_inputs(2, 256, 2, D, 4.0, seed=22, dtype=dtype)
     rng = np.random.default_rng(98)
     h0 = rng.standard_normal(h0.shape).astype(np.float32)
     dhT = rng.standard_normal(h0.shape).astype(np.float32)
