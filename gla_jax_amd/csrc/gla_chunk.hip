@@ -199,9 +199,18 @@ static int chunk_fwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t
     void *prodT = (void *)ws;
     float *decay = (float *)(ws + p.prod);
     unsigned char *pexp = ws + p.prod + p.scale_off;
-    void *statesT = (void *)(ws + p.prod + p.decay);   // [dv][dk], consumed by the output kernel
+    void *ws_states = (void *)(ws + p.prod + p.decay);
     hipStream_t st = (hipStream_t)stream;
     const int N = (int)(T / p.C);
+    // 16-bit data: ONE array of chunk-start states, tiled, read by the output kernel and (as the residual) by the
+    // gradient kernel; without a residual to write it goes to the workspace.  fp32 data: the [dv][dk] copy for the
+    // output kernel in the workspace beside the residual.
+    const bool tiled = dtype == GLA_BF16;
+    void *statesT = tiled ? nullptr : ws_states;
+    void *statesN = tiled && !states ? ws_states : states;
+    const int tail = statesN == states ? 1 : 0;            // the residual has a slot for the final state
+    const void *out_states = tiled ? statesN : statesT;
+    const int slots = tiled ? N + tail : N;
     return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d, auto dm) -> int {
         typedef decltype(t) E;
         constexpr int C_ = decltype(c)::value, D_ = decltype(d)::value, DM_ = decltype(dm)::value;
@@ -212,15 +221,15 @@ static int chunk_fwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t
         if (e) return e;
         if (stages & 2)
             e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 0, hidden_dtype, hidden_init, prodT, decay, pexp,
-                                              statesT, states, hidden_final, 1);
+                                              statesT, statesN, hidden_final, tail, tiled);
         if (e) return e;
         if ((stages & 4) && !wide)
-            e = launch_chunk_out<E, C_, D_, DM_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, statesT,
-                                                 out);
+            e = launch_chunk_out<E, C_, D_, DM_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, out_states,
+                                                 slots, out);
         if ((stages & 4) && wide) {
             if constexpr (sizeof(E) == 2 && D_ == 128 && DM_ == 128)
                 e = launch_chunk_out<E, C_, D_, DM_, true>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query,
-                                                           statesT, out);
+                                                           out_states, slots, out);
             else
                 e = GLA_ERR_UNSUPPORTED;
         }
@@ -350,7 +359,7 @@ static int chunk_bwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t
         if (e) return e;
         if (stages & 2)
             e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 1, hidden_dtype, dhidden_final, prodT, decay, pexp,
-                                              dstatesT, dstatesN, dhidden_init, 0);
+                                              dstatesT, dstatesN, dhidden_init, 0, 0);
         if (e) return e;
         if ((stages & 4) && !wide)
             e = launch_chunk_grad<E, C_, D_, DM_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,

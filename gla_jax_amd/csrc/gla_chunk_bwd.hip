@@ -102,7 +102,7 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             const int idx = threadIdx.x + u * C * 4;
             if (kPieces % (C * 4) == 0 || idx < kPieces) {
                 const int off = (32 * slice + idx / (D / 8)) * D + (idx % (D / 8)) * 8;
-                pfS[u] = ld8_once(Sn + off);
+                pfS[u] = ld8_once(Sn + state_offset<T, D>(32 * slice + idx / (D / 8), (idx % (D / 8)) * 8));
                 pfDn[u] = ld8_once(dSn + off);
                 pfDt[u] = ld8_once(dSt + off);
             }

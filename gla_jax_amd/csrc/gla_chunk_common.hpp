@@ -173,6 +173,16 @@ template <int D, int DM, typename P, typename V> __device__ __forceinline__ void
     if (RowMap<D, DM>::live(c)) st8_once(row_ks + 8 * c, v);
 }
 
+// The chunk states of 16-bit data lie in memory as 32 x 32 tiles, [dk/32][dv/32][32][32] (2 KB each), so that both a
+// slab of 32 key features (all value features) and a slab of 32 value features (all key features) are made of
+// whole tiles: the scan writes ONE array per direction and every consumer reads 2 KB pieces whichever way it
+// contracts.  fp32 states stay row-major (and are written in both orientations).
+template <typename T, int D> __device__ __forceinline__ int state_offset(int dk, int dv)
+{
+    if constexpr (sizeof(T) == 2) return (((dk >> 5) * (D / 32) + (dv >> 5)) << 10) + ((dk & 31) << 5) + (dv & 31);
+    else return dk * D + dv;
+}
+
 // LDS tiles are row-major [rows][D] with a 16-byte pad per row.
 template <typename T, int D> struct TileGeom {
     static constexpr int kStride = D + 16 / (int)sizeof(T);

@@ -26,7 +26,7 @@ namespace gla {
 template <typename T, int C, int D, int DM, bool WIDE>
 __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C / 32))) void chunk_out_kernel(
     const float *__restrict__ g, const T *__restrict__ v, const T *__restrict__ k, const T *__restrict__ q,
-    const T *__restrict__ states, std::conditional_t<WIDE, float, T> *__restrict__ out, int T_len, int H)
+    const T *__restrict__ states, int slots, std::conditional_t<WIDE, float, T> *__restrict__ out, int T_len, int H)
 {
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4;
     constexpr int LS = TileGeom<T, D>::kStride;
@@ -35,7 +35,13 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     extern __shared__ __align__(16) unsigned char smem[];
     T *Vn = reinterpret_cast<T *>(smem);           // [C][LS]       value
     T *Kh = Vn + C * LS;                           // [C - 16][LS]  k * exp(tau_J - l_j), sub-blocks 0 .. NB-2
-    T *St = Kh + (C - 16) * LS;                    // [32][LS]      32 rows of the chunk-start state [dv][dk]
+    T *St = Kh + (C - 16) * LS;                    // [32][LS]      32 rows of the chunk-start state [dv][dk] (fp32 data)
+    // 16-bit data: the slab [all dk][32 dv] of the tiled state, as it lies in memory ([dk][SS]); the products read
+    // it transposed
+    constexpr bool kTiled = sizeof(T) == 2;
+    constexpr int SS = 32;                         // row stride of the slab: the rows as they lie in a tile
+    static_assert(!kTiled || D * SS <= 32 * LS, "the slab fits where the 32 staged rows were");
+    const TrLane<T> Ls = make_tr_lane<T>(SS);
     float *rtab = reinterpret_cast<float *>(St + 32 * LS);   // [NB][D] exp(tau_m)
 
     const int lane = threadIdx.x & 63;
@@ -54,20 +60,29 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
     constexpr int kPieces = 32 * D / 8;                       // 8-element pieces of a slice
     constexpr int kPer = (kPieces + C * 4 - 1) / (C * 4);     // pieces per thread
     D8 pf[kPer];
-    const T *sp = states + (((int64_t)b * H + h) * N + n) * D * D;
+    const T *sp = states + (((int64_t)b * H + h) * slots + n) * D * D;
     auto stage_fetch = [&](int slice) {
 #pragma unroll
         for (int u = 0; u < kPer; ++u) {
             const int idx = threadIdx.x + u * C * 4;
-            if (kPieces % (C * 4) == 0 || idx < kPieces)
-                pf[u] = ld8(sp + (32 * slice + idx / (D / 8)) * D + (idx % (D / 8)) * 8);
+            if (kPieces % (C * 4) == 0 || idx < kPieces) {
+                if constexpr (kTiled)      // tiles (i, slice), i = idx / 128: 2 KB each, read as they lie
+                    pf[u] = ld8(sp + (((idx >> 7) * (D / 32) + slice) << 10) + (idx & 127) * 8);
+                else
+                    pf[u] = ld8(sp + (32 * slice + idx / (D / 8)) * D + (idx % (D / 8)) * 8);
+            }
         }
     };
     auto stage_store = [&]() {
 #pragma unroll
         for (int u = 0; u < kPer; ++u) {
             const int idx = threadIdx.x + u * C * 4;
-            if (kPieces % (C * 4) == 0 || idx < kPieces) st8(St + (idx / (D / 8)) * LS + (idx % (D / 8)) * 8, pf[u]);
+            if (kPieces % (C * 4) == 0 || idx < kPieces) {
+                if constexpr (kTiled)
+                    st8(St + (32 * (idx >> 7) + ((idx & 127) >> 2)) * SS + 8 * (idx & 3), pf[u]);
+                else
+                    st8(St + (idx / (D / 8)) * LS + (idx % (D / 8)) * 8, pf[u]);
+            }
         }
     };
 
@@ -149,9 +164,22 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
         f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
         for (int k2 = 0; k2 < KS; ++k2) {
+            if constexpr (kTiled) {
+                // step (k2, half) contracts over dk = 32 k2 + 8c + 4 half + m, which is what lane (i, c) holds of
+                // (q e^{L})_i; 16 key features per product, the slab read transposed
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-                acc[tt] = mma_d(ld8(St + L.own + 4 * tt * LS + 32 * k2), qb[k2], acc[tt]);
+                for (int half = 0; half < 2; ++half) {
+                    const T4 qh4 = half ? __builtin_shufflevector(qb[k2], qb[k2], 4, 5, 6, 7)
+                                        : __builtin_shufflevector(qb[k2], qb[k2], 0, 1, 2, 3);
+#pragma unroll
+                    for (int tt = 0; tt < 2; ++tt)
+                        acc[tt] = mma_t(lds_tr4(St + Ls.k8 + (32 * k2 + 4 * half) * SS + 4 * tt, SS), qh4, acc[tt]);
+                }
+            } else {
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+                    acc[tt] = mma_d(ld8(St + L.own + 4 * tt * LS + 32 * k2), qb[k2], acc[tt]);
+            }
         }
 #pragma unroll
         for (int J = 0; J < NB; ++J) {
@@ -182,7 +210,7 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
 
 template <typename T, int C, int D, int DM, bool WIDE>
 int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
-                     const void *q, const void *states, void *out)
+                     const void *q, const void *states, int slots, void *out)
 {
     constexpr int LS = TileGeom<T, D>::kStride;
     const size_t lds = (size_t)(2 * C - 16 + 32) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
@@ -191,13 +219,13 @@ int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, co
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(T_len / C * H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, g, (const T *)v, (const T *)k, (const T *)q,
-                       (const T *)states, (std::conditional_t<WIDE, float, T> *)out, T_len, H);
+                       (const T *)states, slots, (std::conditional_t<WIDE, float, T> *)out, T_len, H);
     return launch_status();
 }
 
 #define GLA_INST_OUT_AS(T, C, D, DM, WIDE)                                                                   \
     template int launch_chunk_out<T, C, D, DM, WIDE>(hipStream_t, int, int, int, const float *, const void *, \
-                                                     const void *, const void *, const void *, void *);
+                                                     const void *, const void *, const void *, int, void *);
 #define GLA_INST_OUT(T, C, D, DM) GLA_INST_OUT_AS(T, C, D, DM, false)
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUT)
 GLA_INST_OUT_AS(__bf16, 128, 128, 128, true)

@@ -43,13 +43,15 @@ template <typename T, int D, int DM>
 // hdt = gla_dtype of hin / hout (hidden_init and hidden_final, or their cotangents)
 int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const void *hin, const void *prodT,
                       const float *decay, const unsigned char *pexp, void *statesT, void *statesN, void *hout,
-                      int tail);
+                      int tail, int tiled);
 
 // WIDE (built for bf16 at D = 128 only): `out`, or `dv`, `dk`, `dq`, are float arrays, for the two passes that make
 // up head dimension 256
 template <typename T, int C, int D, int DM, bool WIDE = false>
+// states: the chunk-start states the kernel contracts over dk: for 16-bit data the tiled [dk][dv] array with `slots`
+// states per (b,h) (the residual, or its stand-in in the workspace), for fp32 data the [dv][dk] array of the workspace
 int launch_chunk_out(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,
-                     const void *q, const void *states, void *out);
+                     const void *q, const void *states, int slots, void *out);
 
 template <typename T, int C, int D, int DM, bool WIDE = false>
 int launch_chunk_grad(hipStream_t st, int B, int T_len, int H, const float *g, const void *v, const void *k,

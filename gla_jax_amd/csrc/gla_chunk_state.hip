@@ -203,7 +203,7 @@ __global__ __launch_bounds__(64) void chunk_scan_kernel(const void *__restrict__
                                                          const unsigned char *__restrict__ pexp,
                                                          T *__restrict__ statesT, T *__restrict__ statesN,
                                                          void *__restrict__ hout, int N, int reverse, int tail,
-                                                         int hdt)
+                                                         int hdt, int tiled)
 {
     typedef typename Pair<T>::type P2;
     typedef typename FragTypes<T>::t4 T4;
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(64) void chunk_scan_kernel(const void *__restrict__
     const bool odd = (r & 1) != 0;
     auto emit_n = [&](int64_t slot) {
         T4 t = pack4<T>(f32x4{X[0], X[1], X[2], X[3]});
-        *reinterpret_cast<T4 *>(statesN + sbaseN + slot * D * D + dk * D + dv0) = t;
+        *reinterpret_cast<T4 *>(statesN + sbaseN + slot * D * D + (tiled ? state_offset<T, D>(dk, dv0) : dk * D + dv0)) = t;
     };
     auto emit = [&](int n) {
         if (statesT) {
@@ -338,17 +338,17 @@ int launch_chunk_outer(hipStream_t st, int mode, int B, int T_len, int H, const 
 template <typename T, int D, int DM>
 int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const void *hin, const void *prodT,
                       const float *decay, const unsigned char *pexp, void *statesT, void *statesN, void *hout,
-                      int tail)
+                      int tail, int tiled)
 {
     typedef typename Prod<T>::type P;
     dim3 grid(BH, (D / 16) * (D / 16)), block(64);
     constexpr int kFew = 8;
     if ((int64_t)grid.y * BH >= 1024) {      // at least a wave per SIMD
         hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, kFew>), grid, block, 0, st, hin, (const P *)prodT, decay, pexp,
-                           (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt);
+                           (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt, tiled);
     } else {
         hipLaunchKernelGGL((chunk_scan_kernel<T, D, DM, 16>), grid, block, 0, st, hin, (const P *)prodT, decay, pexp,
-                           (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt);
+                           (T *)statesT, (T *)statesN, hout, N, reverse, tail, hdt, tiled);
     }
     return launch_status();
 }
@@ -358,13 +358,12 @@ int launch_chunk_scan(hipStream_t st, int BH, int N, int reverse, int hdt, const
                                                  const void *, void *, float *, unsigned char *);
 #define GLA_INST_SCAN(T, D, DM)                                                                       \
     template int launch_chunk_scan<T, D, DM>(hipStream_t, int, int, int, int, const void *, const void *, \
-                                             const float *, const unsigned char *, void *, void *, void *, int);
+                                             const float *, const unsigned char *, void *, void *, void *, int, int);
 GLA_FOR_EACH_CHUNK_CONFIG(GLA_INST_OUTER)
 GLA_INST_SCAN(__bf16, 32, 16)
 GLA_INST_SCAN(__bf16, 32, 32)
 GLA_INST_SCAN(__bf16, 64, 64)
 GLA_INST_SCAN(__bf16, 128, 128)
-GLA_INST_SCAN(__bf16, 256, 256)
 GLA_INST_SCAN(float, 32, 16)
 GLA_INST_SCAN(float, 32, 32)
 GLA_INST_SCAN(float, 64, 64)
