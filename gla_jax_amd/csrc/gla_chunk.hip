@@ -359,7 +359,8 @@ static int chunk_bwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t
         if (e) return e;
         if (stages & 2)
             e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 1, hidden_dtype, dhidden_final, prodT, decay, pexp,
-                                              dstatesT, dstatesN, dhidden_init, 0, 0);
+                                              dtype == GLA_BF16 ? nullptr : dstatesT, dstatesN, dhidden_init, 0,
+                                              dtype == GLA_BF16);
         if (e) return e;
         if ((stages & 4) && !wide)
             e = launch_chunk_grad<E, C_, D_, DM_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,

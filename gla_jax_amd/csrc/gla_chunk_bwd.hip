@@ -87,7 +87,12 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
     // ---- staging of the state operands -----------------------------------------------------------------
     // A slice needs rows 32*slice .. +31 of S_n [dk][dv], dS' [dk][dv] and dS' [dv][dk]: 3 x 32 rows of
     // D elements.  They go through registers: requested a slice ahead, written to LDS between two barriers.
+    // 16-bit data: S_n and dS' are single arrays of 32 x 32 tiles (state_offset).  Their 32 rows [dk][all dv] are
+    // staged as rows; the third operand, 32 rows of dS'^T [dv][all dk], is the slab [all dk][32 dv] of the same array,
+    // read as it lies (whole tiles) and transposed on its way into LDS.  fp32 data: dS' comes in both orientations,
+    // row-major.
     T *sS = tV, *sDn = tV + 32 * LS, *sDt = tV + 64 * LS;
+    constexpr bool kTiled = sizeof(T) == 2;
     constexpr int kPieces = 32 * D / 8;                       // 8-element pieces of one staged operand
     constexpr int kPer = (kPieces + C * 4 - 1) / (C * 4);     // pieces per thread
     D8 pfS[kPer], pfDn[kPer], pfDt[kPer];
@@ -102,9 +107,15 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
             const int idx = threadIdx.x + u * C * 4;
             if (kPieces % (C * 4) == 0 || idx < kPieces) {
                 const int off = (32 * slice + idx / (D / 8)) * D + (idx % (D / 8)) * 8;
-                pfS[u] = ld8_once(Sn + state_offset<T, D>(32 * slice + idx / (D / 8), (idx % (D / 8)) * 8));
-                pfDn[u] = ld8_once(dSn + off);
-                pfDt[u] = ld8_once(dSt + off);
+                const int toff = state_offset<T, D>(32 * slice + idx / (D / 8), (idx % (D / 8)) * 8);
+                pfS[u] = ld8_once(Sn + toff);
+                if constexpr (kTiled) {
+                    pfDn[u] = ld8(dSn + toff);    // read again by the workgroup as part of the slabs of other slices
+                    pfDt[u] = ld8(dSn + (((idx >> 7) * (D / 32) + slice) << 10) + (idx & 127) * 8);   // tiles (i, slice)
+                } else {
+                    pfDn[u] = ld8_once(dSn + off);
+                    pfDt[u] = ld8_once(dSt + off);
+                }
             }
         }
     };
@@ -121,7 +132,16 @@ __global__ __launch_bounds__(C * 4) void chunk_grad_kernel(
                 const int row = idx / (D / 8), c8 = (idx % (D / 8)) * 8;
                 st8(sS + row * LS + c8, pfS[u]);
                 st8(sDn + row * LS + c8, pfDn[u]);
-                st8(sDt + row * LS + c8, pfDt[u]);
+                if constexpr (kTiled) {
+                    // the piece holds 8 value features of ONE key feature: it goes to 8 rows of the staged [dv][dk]
+                    // operand, two bytes each (8 KB per slice and workgroup: the transposition costs next to nothing
+                    // here, and the products keep the form and the registers they had)
+                    const int dkk = 32 * (idx >> 7) + ((idx & 127) >> 2), dvv = 8 * (idx & 3);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sDt[(dvv + e) * LS + dkk] = pfDt[u][e];
+                } else {
+                    st8(sDt + row * LS + c8, pfDt[u]);
+                }
                 // chunk-level gate gradient (gla.py:782), first term: e^{L_end} sum_v S_n * dS' per key feature.
                 // (The sum of both terms is sum_v dS' * S_{n+1}; formed that way from the stored S_{n+1} it carries
                 // the rounding of a whole state instead of a decayed one, which cost two sweep cases their bound.)
