@@ -42,7 +42,7 @@ KERNEL_SOURCES = {
 }
 MEASURED_TRAFFIC = {
     # (kernel, B, T, H, D, chunk, source hash): bytes per launch
-    ("chunk_grad_kernel", 4, 4096, 6, 128, 128, "1316e680aa3c"): 408.3e6,
+    ("chunk_grad_kernel", 4, 4096, 6, 128, 128, "7777fc4c77fd"): 394.7e6,
 }
 
 
@@ -170,13 +170,13 @@ def bench_chunk(B, T, H, D, chunk, shift, steps, warmup, public=True):
     # algorithmic bytes (inputs read once, outputs written once) and what each kernel really moves
     kernels = {
         "fwd.chunk_outer_kernel": (lambda: fwd(1), 8 * D * n_th, 8 * D * n_th + prod),
-        # the scans write the chunk states in both orientations; the gradient kernel reads three state
-        # arrays (S_n, dS' twice) and the gates, q and k a second time (once for the score
-        # blocks, once per feature slice; about half of that second read is served by the L2: measured)
-        "fwd.chunk_scan_kernel": (lambda: fwd(2), 0, prod + 2 * state_bf16),
+        # the scans write ONE tiled array of chunk states each; the gradient kernel reads S_n, dS' by rows and dS' by
+        # slabs (the same array a second time), and the gates, q and k a second time (once for the score blocks,
+        # once per feature slice; about half of each second read is served by the L2: measured)
+        "fwd.chunk_scan_kernel": (lambda: fwd(2), 0, prod + state_bf16),
         "fwd.chunk_out_kernel": (lambda: fwd(4), 12 * D * n_th, 12 * D * n_th + state_bf16),
         "bwd.chunk_outer_kernel": (lambda: bwd(1), 8 * D * n_th, 8 * D * n_th + prod),
-        "bwd.chunk_scan_kernel": (lambda: bwd(2), 0, prod + 2 * state_bf16),
+        "bwd.chunk_scan_kernel": (lambda: bwd(2), 0, prod + state_bf16),
         "bwd.chunk_grad_kernel": (lambda: bwd(4), 22 * D * n_th, 26 * D * n_th + 3 * state_bf16),
     }
     per = {}

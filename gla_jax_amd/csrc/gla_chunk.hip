@@ -14,6 +14,7 @@ struct ChunkPlan {
     int D = 0;       // head dimension the kernels work on: DK, or 32 for DK = 16 (rows padded by zeros on the way in)
     size_t prod = 0, decay = 0, states = 0;   // byte sizes, each rounded up to 256
     size_t scale_off = 0;                     // where the products' exponents start inside the decay region
+    int bwd_states = 2;                       // arrays of d(chunk-end state): one (tiled) for 16-bit data, both orientations for fp32
     size_t resid = 0;                         // the forward residual: N + 1 states per (b,h), the last one final
     // Head dimension 256 runs as two passes of the 128-feature kernels over 2H heads (gla_split.hip); the
     // sizes above are then those of one such pass, and:
@@ -28,7 +29,7 @@ struct ChunkPlan {
     size_t fwd_bytes() const { return prod + decay + states + (split ? rows + (wide ? 2 : 1) * rows_f32 + 4 * hid : 0); }
     size_t bwd_bytes() const
     {
-        return prod + decay + 2 * states + (split ? 2 * rows + (wide ? 7 : 4) * rows_f32 + 4 * hid : 0);
+        return prod + decay + bwd_states * states + (split ? 2 * rows + (wide ? 7 : 4) * rows_f32 + 4 * hid : 0);
     }
     size_t resid_bytes() const { return split ? 2 * resid : resid; }
 };
@@ -81,6 +82,7 @@ static int plan_chunk(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, i
     plan->scale_off = (size_t)B * H * N * DK * sizeof(float);
     plan->decay = round256(plan->scale_off + (size_t)B * H * N * (DK * DV / 16));
     plan->states = round256((size_t)B * H * N * DK * DV * esz);
+    plan->bwd_states = dtype == GLA_BF16 ? 1 : 2;
     plan->resid = round256((size_t)B * H * (N + 1) * DK * DV * esz);
     return GLA_OK;
 }
@@ -301,7 +303,7 @@ static int chunk_bwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t
         // into the workspace, from where they are added (those of the value side to the other half of each row).
         if (stages != 7) return GLA_ERR_UNSUPPORTED;
         hipStream_t st = (hipStream_t)stream;
-        const size_t sub = p.prod + p.decay + 2 * p.states;
+        const size_t sub = p.prod + p.decay + p.bwd_states * p.states;
         if (wide) return GLA_ERR_UNSUPPORTED;
         unsigned char *v_sw = ws + sub, *do_sw = v_sw + p.rows, *dg2 = do_sw + p.rows, *dq2 = dg2 + p.rows_f32,
                       *dk2 = dq2 + p.rows_f32, *dv2 = dk2 + p.rows_f32, *dq1 = dv2 + p.rows_f32,
@@ -345,8 +347,9 @@ static int chunk_bwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t
     void *prodT = (void *)ws;
     float *decay = (float *)(ws + p.prod);
     unsigned char *pexp = ws + p.prod + p.scale_off;
-    void *dstatesT = (void *)(ws + p.prod + p.decay);            // d(chunk-end state), [dv][dk]
-    void *dstatesN = (void *)(ws + p.prod + p.decay + p.states); // the same, [dk][dv]
+    // d(chunk-end state): for 16-bit data ONE tiled array, for fp32 data [dv][dk] and [dk][dv]
+    void *dstatesT = dtype == GLA_BF16 ? nullptr : (void *)(ws + p.prod + p.decay);
+    void *dstatesN = (void *)(ws + p.prod + p.decay + (dtype == GLA_BF16 ? 0 : p.states));
     hipStream_t st = (hipStream_t)stream;
     const int N = (int)(T / p.C);
     return dispatch(dtype, p.C, (int)DK, [&](auto t, auto c, auto d, auto dm) -> int {
@@ -359,8 +362,7 @@ static int chunk_bwd_run(void *stream, int stages, int64_t B, int64_t T, int64_t
         if (e) return e;
         if (stages & 2)
             e = launch_chunk_scan<E, D_, DM_>(st, (int)(B * H), N, 1, hidden_dtype, dhidden_final, prodT, decay, pexp,
-                                              dtype == GLA_BF16 ? nullptr : dstatesT, dstatesN, dhidden_init, 0,
-                                              dtype == GLA_BF16);
+                                              dstatesT, dstatesN, dhidden_init, 0, dtype == GLA_BF16);
         if (e) return e;
         if ((stages & 4) && !wide)
             e = launch_chunk_grad<E, C_, D_, DM_>(st, (int)B, (int)T, (int)H, log_fgate, value, key, query, dout,
