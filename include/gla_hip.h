@@ -137,9 +137,9 @@ int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t H, int64_t 
  * states before every chunk and after the last one, [B,H,T/C+1,DK,DV] in the element type, the analogue of
  * the reference's saved `state` (gla.py:548, 729; its last slice is hidden_final, gla.py:720-723).  C is
  * the tile the kernels run with: the largest one built that divides T (the result does not depend on the
- * chunk length, so chunk_size is validated and otherwise not used).  The layout inside is the library's own (at
- * head dimension 256 it is two such arrays for [B,2H] heads of 128 features, one per pass of the 128-feature
- * kernels).  Returns 0 for unsupported arguments. */
+ * chunk length, so chunk_size is validated and otherwise not used).  The layout inside is the library's own (a
+ * 16-bit state lies as 32 x 32 tiles; at head dimension 256 there are two such arrays for [B,2H] heads of 128
+ * features, one per pass of the 128-feature kernels).  Returns 0 for unsupported arguments. */
 size_t gla_chunk_states_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
                               int64_t chunk_size, gla_dtype dtype);
 /* Bytes of scratch needed by gla_chunk_fwd / gla_chunk_bwd (DK == DV in {16, 32, 64, 128, 256}).  Returns 0 for
