@@ -113,8 +113,8 @@ __global__ __launch_bounds__(C * 4) __attribute__((amdgpu_waves_per_eu(C / 32, C
         for (int e = 0; e < 8; ++e) yv[e] *= fast_exp2(sum[e]);
         st8(Yn + (16 * w + r) * LS + d0, pack8<T>(yv));
     }
-    if (w == 0 && r == 0) {
-        // chunk decay e^{L_end}: the total over all sub-blocks
+    if (w == (MODE == 0 ? NB - 1 : 0) && r == 0) {
+        // chunk decay e^{L_end}: the total over all sub-blocks, formed by the wave that has no totals to add above
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const int d0 = 32 * ks + 8 * c;
