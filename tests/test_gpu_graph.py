@@ -24,9 +24,12 @@ def _buffers(B, T, H, D, chunk, dtype):
     return lib, dt, dev, ws_f, ws_b, states
 
 
-def test_chunk_step_replays_from_a_graph():
+@pytest.mark.parametrize("D", [128, 256])
+def test_chunk_step_replays_from_a_graph(D):
+    """D=256 runs as two passes of the 128-feature kernels with copies and sums between them: all of them are
+    kernels on the caller's stream, so the whole sequence records and replays like a single pass."""
     from gla_jax_amd import _lib
-    B, T, H, D, chunk = 2, 512, 2, 128, 128
+    B, T, H, chunk = 2, 512, 2, 128
     dtype = torch.bfloat16
     lib, dt, (h0, g, v, k, q, dhT, dout), ws_f, ws_b, states = _buffers(B, T, H, D, chunk, dtype)
     outs = lambda: [torch.empty_like(h0), torch.empty_like(v), torch.empty_like(h0), torch.empty_like(g),
@@ -92,6 +95,52 @@ def test_recurrent_step_replays_from_a_graph(D):
     for it in range(3):
         for t in replayed:
             t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("hidden_final", "out", "dh0", "dg", "dv", "dk", "dq"), eager, replayed):
+            assert torch.equal(a, b), f"replay {it}: {name} differs from the eager result"
+
+
+def test_recurrent_step_with_a_workspace_replays_from_a_graph():
+    """Head dimension 256 through gla_recurrent_fwd_ws / gla_recurrent_bwd_ws (two passes of the D=128 matrix-core
+    kernels, their partial results in the caller's workspace)."""
+    from gla_jax_amd import _lib
+    lib = _lib.load()
+    B, T, H, D = 2, 150, 2, 256
+    dtype, dt = torch.bfloat16, _lib.GLA_BF16
+    (h0n, gn, vn, kn, qn), (h0, g, v, k, q) = gpu_inputs(B, T, H, D, 3.0, seed=79, dtype=dtype)
+    dhTn, doutn = cotangents(h0n, vn, 11, dtype)
+    dhT, dout = to_dev(dhTn, dtype), to_dev(doutn, dtype)
+    u8 = lambda n: torch.empty(n, dtype=torch.uint8, device="cuda")
+    ws_f = u8(lib.gla_recurrent_fwd_workspace_bytes(B, T, H, D, D, dt))
+    ws_b = u8(lib.gla_recurrent_bwd_workspace_bytes(B, T, H, D, D, dt))
+    assert ws_f.numel() > 0 and ws_b.numel() > 0
+    outs = lambda: [torch.empty_like(h0), torch.empty_like(v), torch.empty_like(h0), torch.empty_like(g),
+                    torch.empty_like(v), torch.empty_like(k), torch.empty_like(q)]
+    p = lambda t: t.data_ptr()
+
+    def step(stream, o):
+        hT, out, dh0, dg, dv, dk, dq = o
+        _lib.check("gla_recurrent_fwd_ws", lib.gla_recurrent_fwd_ws(stream, B, T, H, D, D, dt, dt, dt, 0, p(h0), p(g),
+                                                                    p(v), p(k), p(q), p(hT), p(out), p(ws_f),
+                                                                    ws_f.numel()))
+        _lib.check("gla_recurrent_bwd_ws", lib.gla_recurrent_bwd_ws(stream, B, T, H, D, D, dt, dt, dt, 0, p(h0), p(g),
+                                                                    p(v), p(k), p(q), p(hT), p(dhT), p(dout), p(dh0),
+                                                                    p(dg), p(dv), p(dk), p(dq), p(ws_b), ws_b.numel()))
+
+    eager = outs()
+    step(torch.cuda.current_stream().cuda_stream, eager)
+    torch.cuda.synchronize()
+    replayed = outs()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(torch.cuda.current_stream().cuda_stream, replayed)
+    for it in range(3):
+        for t in replayed:
+            t.fill_(float("nan"))
+        ws_f.fill_(255)                                       # the workspace holds nothing a replay relies on
+        ws_b.fill_(255)
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
