@@ -215,14 +215,21 @@ def bench_recurrent(B, T, H, D, shift, steps, warmup):
     st = torch.cuda.current_stream().cuda_stream
     p = lambda t: t.data_ptr()
 
+    # the entry points with a workspace: it is empty at this workload's 256 sequences (they run whole, one per compute
+    # unit) and lets shapes with few sequences run as segments side by side
+    n_f = lib.gla_recurrent_fwd_workspace_bytes(B, T, H, D, D, dt)
+    n_b = lib.gla_recurrent_bwd_workspace_bytes(B, T, H, D, D, dt)
+    ws_f = torch.empty(max(n_f, 16), dtype=torch.uint8, device="cuda")
+    ws_b = torch.empty(max(n_b, 16), dtype=torch.uint8, device="cuda")
+
     def fwd():
-        _lib.check("gla_recurrent_fwd", lib.gla_recurrent_fwd(st, B, T, H, D, D, dt, dt, dt, 0, p(h0), p(g), p(v),
-                                                            p(k), p(q), p(hT), p(out)))
+        _lib.check("gla_recurrent_fwd_ws", lib.gla_recurrent_fwd_ws(st, B, T, H, D, D, dt, dt, dt, 0, p(h0), p(g), p(v),
+                                                                    p(k), p(q), p(hT), p(out), p(ws_f), n_f))
 
     def bwd():
-        _lib.check("gla_recurrent_bwd", lib.gla_recurrent_bwd(st, B, T, H, D, D, dt, dt, dt, 0, p(h0), p(g), p(v),
-                                                            p(k), p(q), p(hT), p(dhT), p(dout), p(dh0), p(dg),
-                                                            p(dv), p(dk), p(dq)))
+        _lib.check("gla_recurrent_bwd_ws", lib.gla_recurrent_bwd_ws(st, B, T, H, D, D, dt, dt, dt, 0, p(h0), p(g), p(v),
+                                                                    p(k), p(q), p(hT), p(dhT), p(dout), p(dh0), p(dg),
+                                                                    p(dv), p(dk), p(dq), p(ws_b), n_b))
 
     def step():
         fwd()

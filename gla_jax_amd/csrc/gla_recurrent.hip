@@ -10,6 +10,7 @@
 #include "gla_common.hpp"
 #include "gla_recurrent_stream.hpp"
 #include "gla_split.hpp"
+#include "gla_timesplit.hpp"
 
 namespace gla {
 
@@ -534,39 +535,78 @@ extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, 
                              value, key, query, hidden_final, out);
 }
 
+// ---- a sequence as S segments side by side (gla_timesplit.hip) -------------------------------------------------
+// With fewer (batch, head) pairs than a quarter of the GPU's compute units, a call with a workspace runs every
+// sequence as S segments at once: one pass from zero states for the segments' own contributions, a scan over the
+// segments, and the real pass with the states that enter each segment (fp32); the backward does the same for
+// the states' cotangents.  The segments are batch entries of the same kernels: [B,T,H,D] is [B*S,T/S,H,D].
+namespace gla {
+constexpr int64_t kComputeUnits = 256;       // MI355X
+constexpr int64_t kMinSegment = 256;         // steps: below this the extra pass costs more than the idle units
+struct TimeSplit {
+    int64_t S = 1, L = 0;
+    size_t hid = 0, sums = 0;
+    TimeSplit(int64_t B, int64_t T, int64_t H, int64_t DK, int dtype)
+    {
+        const int64_t seqs = B * H * (DK == 256 ? 2 : 1);    // head dimension 256 runs as 2H heads of 128
+        while (seqs * S * 2 <= kComputeUnits && T % (S * 2) == 0 && T / (S * 2) >= kMinSegment && B * S * 2 <= 65535)
+            S *= 2;
+        // Two segments mean two passes over half the steps each: that pays only where the first pass is the lean one
+        // (bf16 data) and the kernels are heavy (128 features: 1.47 -> 1.32 ms at B16 T2048 H8; 64 features:
+        // 0.43 -> 0.45 ms).  From four segments on it pays everywhere.
+        if (S < (dtype == GLA_BF16 && DK >= 128 ? 2 : 4)) S = 1;
+        L = T / S;
+        hid = SplitSizes::round_up256((size_t)B * S * H * DK * DK * 4);
+        sums = SplitSizes::round_up256((size_t)B * S * H * DK * 4);
+    }
+    bool on() const { return S > 1; }
+    // forward: entering states, the segments' own contributions, gate sums
+    size_t fwd() const { return on() ? 2 * hid + sums : 0; }
+    // backward: the same and the entering cotangents
+    size_t bwd() const { return on() ? 3 * hid + sums : 0; }
+};
+static size_t inner_fwd_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int dtype)
+{
+    return DK == 256 ? SplitSizes(B, T, H, dtype).fwd() : 0;
+}
+static size_t inner_bwd_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int dtype)
+{
+    return DK == 256 ? SplitSizes(B, T, H, dtype).bwd() : 0;
+}
+}  // namespace gla
+
 extern "C" size_t gla_recurrent_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
                                                     gla_dtype dtype)
 {
-    if (gla::check_recurrent(B, T, H, DK, DV, dtype, GLA_F32, GLA_F32) || DK != 256 || 2 * H > 65535) return 0;
-    return gla::SplitSizes(B, T, H, dtype).fwd();
+    if (gla::check_recurrent(B, T, H, DK, DV, dtype, GLA_F32, GLA_F32) || 2 * H > 65535) return 0;
+    const gla::TimeSplit ts(B, T, H, DK, dtype);      // the passes run on B*S batch entries of L steps: their state blocks count
+    return ts.fwd() + gla::inner_fwd_bytes(B * ts.S, ts.L, H, DK, dtype);
 }
 
 extern "C" size_t gla_recurrent_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
                                                     gla_dtype dtype)
 {
-    if (gla::check_recurrent(B, T, H, DK, DV, dtype, GLA_F32, GLA_F32) || DK != 256 || 2 * H > 65535) return 0;
-    return gla::SplitSizes(B, T, H, dtype).bwd();
+    if (gla::check_recurrent(B, T, H, DK, DV, dtype, GLA_F32, GLA_F32) || 2 * H > 65535) return 0;
+    const gla::TimeSplit ts(B, T, H, DK, dtype);
+    return ts.bwd() + gla::inner_bwd_bytes(B * ts.S, ts.L, H, DK, dtype);
 }
 
-extern "C" int gla_recurrent_fwd_ws(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                                    gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
-                                    const void *hidden_init, const float *log_fgate, const void *value,
-                                    const void *key, const void *query, void *hidden_final, void *out,
-                                    void *workspace, size_t workspace_bytes)
+// One pass over whole sequences; arguments checked by the caller.  Head dimension 256 with a workspace: two passes
+// of the 128-feature kernels; everything else: the kernels directly.
+static int recurrent_fwd_inner(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, gla_dtype dtype,
+                               gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse, const void *hidden_init,
+                               const float *log_fgate, const void *value, const void *key, const void *query,
+                               void *hidden_final, void *out, void *workspace, bool state_only = false)
 {
-    const size_t need = gla_recurrent_fwd_workspace_bytes(B, T, H, DK, DV, dtype);
-    if (!need)      // every other head dimension needs no workspace
+    // state_only: the caller wants hidden_final alone and `out` is a buffer it will overwrite.  The matrix-core
+    // kernels have a form without the output products; the other kernels write the unused `out`.
+    const bool lean = state_only && dtype == GLA_BF16;
+    if (lean && (DK == 64 || DK == 128))
+        return gla::launch_recurrent_stream_state((hipStream_t)stream, B, T, H, DK, reverse, hidden_dtype, hidden_init,
+                                                  log_fgate, value, key, query, hidden_final);
+    if (DK != 256 || !workspace)
         return recurrent_fwd_run(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
                                  log_fgate, value, key, query, hidden_final, out);
-    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, hidden_dtype, out_dtype);
-    if (rc) return rc;
-    const void *ptrs[] = {hidden_init, log_fgate, value, key, query, hidden_final, out};
-    for (const void *p : ptrs) {
-        if (!p) return GLA_ERR_NULL;
-        if (!gla::aligned16(p)) return GLA_ERR_ALIGN;
-    }
-    if (!workspace || workspace_bytes < need) return GLA_ERR_WORKSPACE;
-    if (!gla::aligned16(workspace)) return GLA_ERR_ALIGN;
     const gla::SplitSizes z(B, T, H, dtype);
     hipStream_t st = (hipStream_t)stream;
     unsigned char *ws = (unsigned char *)workspace;
@@ -578,6 +618,15 @@ extern "C" int gla_recurrent_fwd_ws(void *stream, int64_t B, int64_t T, int64_t 
     if (e) return e;
     // key half a with value half a on the arrays as they lie, then key half a with the other value half; `out` of
     // both in fp32 (the recurrent_gla_naive flavour of the 128-feature kernels)
+    if (lean) {
+        e = gla::launch_recurrent_stream_state(st, B, T, 2 * H, 128, reverse, hidden_dtype, h0_same, log_fgate, value, key,
+                                               query, hT_same);
+        if (e) return e;
+        e = gla::launch_recurrent_stream_state(st, B, T, 2 * H, 128, reverse, hidden_dtype, h0_cross, log_fgate, v_sw, key,
+                                               query, hT_cross);
+        if (e) return e;
+        return gla::launch_hidden_blocks(st, hidden_dtype, B * H, hidden_final, hT_same, hT_cross, 0);
+    }
     e = recurrent_fwd_run(stream, B, T, 2 * H, 128, 128, dtype, hidden_dtype, GLA_F32, reverse, h0_same, log_fgate,
                           value, key, query, hT_same, out1);
     if (e) return e;
@@ -587,6 +636,48 @@ extern "C" int gla_recurrent_fwd_ws(void *stream, int64_t B, int64_t T, int64_t 
     e = gla::launch_sum_rows(st, out_dtype, B * T * H, out, (const float *)out1, (const float *)out2, 1);
     if (e) return e;
     return gla::launch_hidden_blocks(st, hidden_dtype, B * H, hidden_final, hT_same, hT_cross, 0);
+}
+
+extern "C" int gla_recurrent_fwd_ws(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                    gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
+                                    const void *hidden_init, const float *log_fgate, const void *value,
+                                    const void *key, const void *query, void *hidden_final, void *out,
+                                    void *workspace, size_t workspace_bytes)
+{
+    const size_t need = gla_recurrent_fwd_workspace_bytes(B, T, H, DK, DV, dtype);
+    if (!need)      // nothing to gain from a workspace at this shape
+        return recurrent_fwd_run(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
+                                 log_fgate, value, key, query, hidden_final, out);
+    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, hidden_dtype, out_dtype);
+    if (rc) return rc;
+    const void *ptrs[] = {hidden_init, log_fgate, value, key, query, hidden_final, out};
+    for (const void *p : ptrs) {
+        if (!p) return GLA_ERR_NULL;
+        if (!gla::aligned16(p)) return GLA_ERR_ALIGN;
+    }
+    if (!workspace || workspace_bytes < need) return GLA_ERR_WORKSPACE;
+    if (!gla::aligned16(workspace)) return GLA_ERR_ALIGN;
+    const gla::TimeSplit ts(B, T, H, DK, dtype);
+    if (!ts.on())
+        return recurrent_fwd_inner(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
+                                   log_fgate, value, key, query, hidden_final, out, workspace);
+    hipStream_t st = (hipStream_t)stream;
+    unsigned char *ws = (unsigned char *)workspace;
+    float *entering = (float *)ws, *loc = (float *)(ws + ts.hid), *sums = (float *)(ws + 2 * ts.hid);
+    void *inner_ws = DK == 256 ? ws + ts.fwd() : nullptr;
+    int e = gla::launch_zero_fill(st, entering, ts.hid);
+    if (e) return e;
+    e = gla::launch_segment_gate_sums(st, B, ts.S, ts.L, H, (int)DK, log_fgate, sums);
+    if (e) return e;
+    // every segment from a zero state: its own contribution to the state that leaves it (`out` is written again below)
+    e = recurrent_fwd_inner(stream, B * ts.S, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, entering, log_fgate,
+                            value, key, query, loc, out, inner_ws, true);
+    if (e) return e;
+    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, hidden_init, loc, sums, nullptr, 0,
+                                 reverse, entering, hidden_final);
+    if (e) return e;
+    return recurrent_fwd_inner(stream, B * ts.S, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, entering,
+                               log_fgate, value, key, query, loc, out, inner_ws);
 }
 
 // wide != 0: dvalue, dkey, dquery are float arrays whatever `dtype` is
@@ -630,29 +721,18 @@ extern "C" int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, 
                              dkey, dquery, 0);
 }
 
-extern "C" int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
-                                    gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
-                                    const void *hidden_init, const float *log_fgate, const void *value,
-                                    const void *key, const void *query, const void *hidden_final,
-                                    const void *dhidden_final, const void *dout, void *dhidden_init,
-                                    float *dlog_fgate, void *dvalue, void *dkey, void *dquery, void *workspace,
-                                    size_t workspace_bytes)
+// One backward over whole sequences; arguments checked by the caller (see recurrent_fwd_inner).
+static int recurrent_bwd_inner(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, gla_dtype dtype,
+                               gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse, const void *hidden_init,
+                               const float *log_fgate, const void *value, const void *key, const void *query,
+                               const void *hidden_final, const void *dhidden_final, const void *dout,
+                               void *dhidden_init, float *dlog_fgate, void *dvalue, void *dkey, void *dquery,
+                               void *workspace)
 {
-    const size_t need = gla_recurrent_bwd_workspace_bytes(B, T, H, DK, DV, dtype);
-    if (!need)
+    if (DK != 256 || !workspace)
         return recurrent_bwd_run(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
                                  log_fgate, value, key, query, hidden_final, dhidden_final, dout, dhidden_init,
                                  dlog_fgate, dvalue, dkey, dquery, 0);
-    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, hidden_dtype, out_dtype);
-    if (rc) return rc;
-    const void *ptrs[] = {hidden_init, log_fgate, value, key, query, hidden_final, dhidden_final,
-                          dout, dhidden_init, dlog_fgate, dvalue, dkey, dquery};
-    for (const void *p : ptrs) {
-        if (!p) return GLA_ERR_NULL;
-        if (!gla::aligned16(p)) return GLA_ERR_ALIGN;
-    }
-    if (!workspace || workspace_bytes < need) return GLA_ERR_WORKSPACE;
-    if (!gla::aligned16(workspace)) return GLA_ERR_ALIGN;
     const gla::SplitSizes z(B, T, H, dtype);
     hipStream_t st = (hipStream_t)stream;
     unsigned char *ws = (unsigned char *)workspace;
@@ -686,4 +766,76 @@ extern "C" int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t 
     e = gla::launch_add_rows(st, GLA_F32, rows, dlog_fgate, dg2, 0);
     if (e) return e;
     return gla::launch_hidden_blocks(st, hidden_dtype, B * H, dhidden_init, dh0_same, dh0_cross, 0);
+}
+
+extern "C" int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
+                                    gla_dtype dtype, gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse,
+                                    const void *hidden_init, const float *log_fgate, const void *value,
+                                    const void *key, const void *query, const void *hidden_final,
+                                    const void *dhidden_final, const void *dout, void *dhidden_init,
+                                    float *dlog_fgate, void *dvalue, void *dkey, void *dquery, void *workspace,
+                                    size_t workspace_bytes)
+{
+    const size_t need = gla_recurrent_bwd_workspace_bytes(B, T, H, DK, DV, dtype);
+    if (!need)
+        return recurrent_bwd_run(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
+                                 log_fgate, value, key, query, hidden_final, dhidden_final, dout, dhidden_init,
+                                 dlog_fgate, dvalue, dkey, dquery, 0);
+    int rc = gla::check_recurrent(B, T, H, DK, DV, dtype, hidden_dtype, out_dtype);
+    if (rc) return rc;
+    const void *ptrs[] = {hidden_init, log_fgate, value, key, query, hidden_final, dhidden_final,
+                          dout, dhidden_init, dlog_fgate, dvalue, dkey, dquery};
+    for (const void *p : ptrs) {
+        if (!p) return GLA_ERR_NULL;
+        if (!gla::aligned16(p)) return GLA_ERR_ALIGN;
+    }
+    if (!workspace || workspace_bytes < need) return GLA_ERR_WORKSPACE;
+    if (!gla::aligned16(workspace)) return GLA_ERR_ALIGN;
+    const gla::TimeSplit ts(B, T, H, DK, dtype);
+    // The pass for the states' cotangents reads dout where the forward kernels read value, so dout must have value's
+    // type: with an fp32 dout beside bf16 data (the recurrent_gla_naive flavour) the sequences run whole.
+    if (!ts.on() || out_dtype != dtype)
+        return recurrent_bwd_inner(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
+                                   log_fgate, value, key, query, hidden_final, dhidden_final, dout, dhidden_init,
+                                   dlog_fgate, dvalue, dkey, dquery, DK == 256 ? (unsigned char *)workspace + ts.bwd() : nullptr);
+    hipStream_t st = (hipStream_t)stream;
+    unsigned char *ws = (unsigned char *)workspace;
+    float *entering = (float *)ws, *loc = (float *)(ws + ts.hid), *dleaving = (float *)(ws + 2 * ts.hid),
+          *sums = (float *)(ws + 3 * ts.hid);
+    void *inner_ws = DK == 256 ? ws + ts.bwd() : nullptr;      // sized for the backward, which needs more
+    const int64_t BS = B * ts.S;
+    // 1. the states that enter the segments, as the forward formed them; the pass's `out` lands in dquery, which the
+    //    backward proper overwrites
+    int e = gla::launch_zero_fill(st, entering, ts.hid);
+    if (e) return e;
+    e = gla::launch_segment_gate_sums(st, B, ts.S, ts.L, H, (int)DK, log_fgate, sums);
+    if (e) return e;
+    e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, entering, log_fgate, value,
+                            key, query, loc, dquery, inner_ws, true);
+    if (e) return e;
+    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, hidden_init, loc, sums, nullptr, 0, reverse,
+                                 entering, nullptr);
+    if (e) return e;
+    // 2. the cotangents of the states that leave the segments.  d(state) obeys the state's recurrence against time
+    //    with query for key and dout for value, the decay between two steps being the later step's gate: the same
+    //    forward kernels in the other direction on the gates moved by one row (kept in dlog_fgate until the
+    //    backward proper writes there; the pass's `out` lands in dkey).
+    e = gla::launch_shift_rows(st, B, T, H * DK, log_fgate, dlog_fgate, reverse ? -1 : 1);
+    if (e) return e;
+    e = gla::launch_zero_fill(st, dleaving, ts.hid);
+    if (e) return e;
+    e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, !reverse, dleaving, dlog_fgate, dout,
+                            query, key, loc, dkey, inner_ws, true);
+    if (e) return e;
+    // what enters segment p from the steps behind it: the gate of p's first step (in the order of the recurrence)
+    // times its own contribution, plus its whole decay times what entered from further behind; after the last
+    // segment that is dhidden_init
+    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, dhidden_final, loc, sums, log_fgate,
+                                 reverse ? (int)ts.L - 1 : 0, !reverse, dleaving, dhidden_init);
+    if (e) return e;
+    // 3. the backward proper, every segment with its entering state and its leaving cotangent: the gate gradient's
+    //    running sum starts from sum_v d(state) * state at the segment's end, which is what the steps behind it add
+    return recurrent_bwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, entering, log_fgate,
+                               value, key, query, hidden_final, dleaving, dout, loc, dlog_fgate, dvalue, dkey, dquery,
+                               inner_ws);
 }

@@ -30,7 +30,10 @@ template <> struct OutPack<float> {
     static __device__ __forceinline__ void store(float *p, const float *o) { st8(p, pack8<float>(o)); }
 };
 
-template <typename TO, int C, int D>
+// STATE: only hidden_final is wanted (a segment's own contribution to the state, or to its cotangent, when a
+// sequence runs as segments side by side): the scores of earlier sub-blocks, the output products and the stores
+// of `out` are left out, and so is the copy of the state that those products read.
+template <typename TO, int C, int D, bool STATE = false>
 __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
     const void *__restrict__ h0, const float *__restrict__ g, const __bf16 *__restrict__ v,
     const __bf16 *__restrict__ k, const __bf16 *__restrict__ q, void *__restrict__ hT,
@@ -89,7 +92,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
                     Sl[(16 * (wv + i * NDV) + 4 * c + e) * LS + 16 * (nt0 + nt) + r] = (T)(S[i][nt][e] - (float)hi);
                 }
     };
-    publish_state();
+    if constexpr (!STATE) publish_state();
 
     // inputs of the wave's 16 steps of a block, one block ahead
     f32x8 gN[KS];
@@ -141,6 +144,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
         }
         __syncthreads();                     // tiles of this block and the published state are in place
 
+        if constexpr (!STATE) {
         // ---- earlier sub-blocks J < w, walking the q side down; scores kept as packed MFMA operands ----
         // (operands and scores as bf16 head + remainder: the products keep 16 bits of mantissa)
         T4 sc[NB], sl[NB];
@@ -213,6 +217,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
             for (int e = 0; e < 8; ++e) o[e] = acc[e >> 2][e & 3];
             if (valid) OutPack<TO>::store(out + row + fo + 8 * c, o);
         }
+        }   // !STATE
 
         // The next block's rows are requested only here: the registers that receive them are not held through
         // the score and output phases above, and the update below is long enough for them to arrive.
@@ -237,7 +242,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
             }
         }
         __syncthreads();                     // every wave is done with the tiles and the old state
-        publish_state();
+        if constexpr (!STATE) publish_state();
     }
 
 #pragma unroll
@@ -249,14 +254,14 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
         }
 }
 
-template <typename TO, int C, int D>
+template <typename TO, int C, int D, bool STATE = false>
 static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, int hdt, const void *h0, const float *g,
                       const void *v, const void *k, const void *q, void *hT, void *out)
 {
     typedef __bf16 T;
     constexpr int LS = TileGeom<T, D>::kStride;
     const size_t lds = (size_t)(3 * C + 2 * D) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
-    auto kern = recurrent_stream_fwd_kernel<TO, C, D>;
+    auto kern = recurrent_stream_fwd_kernel<TO, C, D, STATE>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
@@ -272,6 +277,14 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
 {
     if (D == 64) return launch_one<TO, 128, 64>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, out);
     if (D == 128) return launch_one<TO, 64, 128>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, out);
+    return GLA_ERR_UNSUPPORTED;
+}
+
+int launch_recurrent_stream_state(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, const void *h0,
+                                 const float *g, const void *v, const void *k, const void *q, void *hT)
+{
+    if (D == 64) return launch_one<__bf16, 128, 64, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, nullptr);
+    if (D == 128) return launch_one<__bf16, 64, 128, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, nullptr);
     return GLA_ERR_UNSUPPORTED;
 }
 

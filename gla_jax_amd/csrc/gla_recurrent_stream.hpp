@@ -12,6 +12,10 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
                                 const void *h0, const float *g, const void *v, const void *k, const void *q,
                                 void *hT, void *out);
 
+// The forward without its outputs: hidden_final alone (what a segment contributes to the state that leaves it).
+int launch_recurrent_stream_state(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, const void *h0,
+                                 const float *g, const void *v, const void *k, const void *q, void *hT);
+
 // Sweep 1 of the backward: dq, and q*dq in fp32 into `qdq` (the last step's carries sum_v dhT * (final state)
 // on top).  dout_f32 != 0: `dout` is float (the recurrent_gla_naive flavour), else bf16.  wide != 0 (head dimension
 // 128 only): `dq` is a float array, for the two passes that make up head dimension 256.

@@ -1,0 +1,25 @@
+// recurrent_gla on few sequences: the small kernels that let a sequence run as S segments side by side
+// (gla_timesplit.hip; the entry points that use them are in gla_recurrent.hip).
+#pragma once
+
+#include "gla_common.hpp"
+
+namespace gla {
+
+// sums[b][p][h][d] = sum of g[b][p*L + t][h][d] over the L rows of segment p.  g: [B][S*L][H][D] floats.
+int launch_segment_gate_sums(hipStream_t st, int64_t B, int64_t S, int64_t L, int64_t H, int D, const float *g,
+                             float *sums);
+// dst[b][t] = src[b][t + dir] (dir = +1 or -1) for rows that exist, zeros for the one row per batch entry that has no
+// such neighbour.  Rows are [H*D] floats, T rows per batch entry.
+int launch_shift_rows(hipStream_t st, int64_t B, int64_t T, int64_t row_len, const float *src, float *dst, int dir);
+// The recurrence over segments, elementwise over a [D][D] state per (b, h):
+//     x <- exp(sums[b][p][h][dk]) * x + exp(edge) * loc[b][p][h][dk][dv],       p ascending, or descending from S-1,
+// with entering[b][p] = x before segment p's update (fp32) and `final` = x after the last one (type hdt; may be
+// null).  x starts as init[b][h] (type hdt).  edge = g[b][p*L + edge_row][h][dk] when g is given, else 0.
+int launch_segment_scan(hipStream_t st, int64_t B, int64_t S, int64_t L, int64_t H, int D, int hdt, const void *init,
+                        const float *loc, const float *sums, const float *g, int edge_row, int descending,
+                        float *entering, void *final);
+// n bytes of zeros (a multiple of 16, the address aligned to 16)
+int launch_zero_fill(hipStream_t st, void *dst, size_t n);
+
+}  // namespace gla

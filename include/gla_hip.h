@@ -109,13 +109,23 @@ int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK,
                       const void *dhidden_final, const void *dout,
                       void *dhidden_init, float *dlog_fgate, void *dvalue, void *dkey, void *dquery);
 
-/* The same two rules (gla.py:99-170, 172-269) with a caller-provided workspace.  At head dimension 256 the
- * recurrence then runs as four problems of head dimension 128 (it is a sum over key features and independent over
- * value features): two passes of the 128-feature kernels over 2H heads, on the matrix cores for bf16 data, with
- * the passes' results kept in fp32 in the workspace and rounded once.  Without a workspace (the two entry points
- * above) head dimension 256 runs on per-timestep vector kernels, an order of magnitude slower.  The size
- * functions return 0 where no workspace is needed; the entry points then ignore `workspace` (NULL is fine) and
- * behave exactly like the ones above.  Same results within the tolerance either way. */
+/* The same two rules (gla.py:99-170, 172-269) with a caller-provided workspace, which buys two things.
+ * (1) At head dimension 256 the recurrence runs as four problems of head dimension 128 (it is a sum over key
+ * features and independent over value features): two passes of the 128-feature kernels over 2H heads, on the
+ * matrix cores for bf16 data, with the passes' results kept in fp32 in the workspace and rounded once.  Without a
+ * workspace (the two entry points above) head dimension 256 runs on per-timestep vector kernels, an order of
+ * magnitude slower.
+ * (2) With few sequences (B*H, at head dimension 256 2*B*H, at most a quarter of the GPU's 256 compute units) and
+ * T a multiple of S >= 4 segments of at least 256 steps, every sequence runs as S segments side by side: the
+ * recurrence is linear in the state, so one pass from zero states gives each segment's own contribution, a scan
+ * over the segments the state that enters each (fp32, in the workspace), and a second pass the outputs; the
+ * backward does the same for the states' cotangents first.  One workgroup walks one (batch, head) pair, so without
+ * this a call with 8 pairs uses 8 of 256 compute units.  The backward keeps the gates moved by one row in
+ * dlog_fgate and two passes' unused `out` in dquery and dkey until it writes its results there; with an fp32 dout
+ * beside bf16 data (out_dtype != dtype) it runs the sequences whole.
+ * The size functions return 0 where a workspace buys nothing; the entry points then ignore `workspace` (NULL is
+ * fine) and behave exactly like the ones above.  Same results within the tolerance either way (segments: the
+ * same but for the order of fp32 sums). */
 size_t gla_recurrent_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, gla_dtype dtype);
 size_t gla_recurrent_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, gla_dtype dtype);
 int gla_recurrent_fwd_ws(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,

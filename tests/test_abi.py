@@ -85,14 +85,24 @@ def test_chunk_plan_and_sizes():
     assert sub + 16 * rows + hid <= lib.gla_chunk_bwd_workspace_bytes(B, T, H, 256, 256, 128, _lib.GLA_BF16) <= (
         sub + 16 * rows + hid + 12 * 256)
     assert lib.gla_chunk_states_bytes(B, T, H, 512, 512, 128, _lib.GLA_BF16) == 0
-    # recurrent_gla: a workspace at head dimension 256 only (both passes' results in fp32 and the exchanged rows)
+    # recurrent_gla: a workspace at head dimension 256 (both passes' results in fp32 and the exchanged rows) and, at
+    # every head dimension, where the sequences are few enough to run as S >= 4 segments of >= 256 steps side by
+    # side (B*H*S <= 256 workgroups; S = 2 already for bf16 data at head dimensions 128 and 256): the segments'
+    # states in fp32, twice (backward: three times), and their gate sums
+    r256 = lambda x: (x + 255) & ~255
     for D in (16, 32, 64, 128):
-        assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, D, D, _lib.GLA_BF16) == 0
-        assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, D, D, _lib.GLA_F32) == 0
+        assert lib.gla_recurrent_fwd_workspace_bytes(16, 2048, 16, D, D, _lib.GLA_BF16) == 0    # 256 sequences
+        assert lib.gla_recurrent_bwd_workspace_bytes(16, 2048, 8, D, D, _lib.GLA_F32) == 0      # 128: S would be 2
+        assert lib.gla_recurrent_fwd_workspace_bytes(1, 500, 2, D, D, _lib.GLA_BF16) == 0       # segments below 256 steps
+        two = lib.gla_recurrent_fwd_workspace_bytes(16, 2048, 8, D, D, _lib.GLA_BF16)           # 128 sequences: S = 2
+        assert two == (2 * r256(16 * 2 * 8 * D * D * 4) + r256(16 * 2 * 8 * D * 4) if D == 128 else 0)
+        S = 8                                                                                   # 24 sequences of 4096 steps
+        hid, sums = r256(B * S * H * D * D * 4), r256(B * S * H * D * 4)
+        assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, D, D, _lib.GLA_BF16) == 2 * hid + sums
+        assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, D, D, _lib.GLA_F32) == 3 * hid + sums
+    assert lib.gla_recurrent_fwd_workspace_bytes(1, 1024, 64, 64, 64, _lib.GLA_BF16) == 2 * r256(4 * 64 * 64 * 64 * 4) + (
+        r256(4 * 64 * 64 * 4))                                                                  # S = 4, the smallest
     rows32 = B * T * H * 256 * 4
-    assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, 256, 256, _lib.GLA_BF16) >= rows32 // 2 + 2 * rows32
-    assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, 256, 256, _lib.GLA_BF16) >= rows32 // 2 + 8 * rows32
-    assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, 256, 256, _lib.GLA_F32) >= 9 * rows32
     assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, 256, 128, _lib.GLA_BF16) == 0      # DK != DV: unsupported
 
 

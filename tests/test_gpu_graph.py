@@ -102,12 +102,13 @@ def test_recurrent_step_replays_from_a_graph(D):
             assert torch.equal(a, b), f"replay {it}: {name} differs from the eager result"
 
 
-def test_recurrent_step_with_a_workspace_replays_from_a_graph():
-    """Head dimension 256 through gla_recurrent_fwd_ws / gla_recurrent_bwd_ws (two passes of the D=128 matrix-core
-    kernels, their partial results in the caller's workspace)."""
+@pytest.mark.parametrize("B,T,H,D", [(2, 150, 2, 256), (1, 1024, 2, 64), (1, 1024, 1, 256)])
+def test_recurrent_step_with_a_workspace_replays_from_a_graph(B, T, H, D):
+    """gla_recurrent_fwd_ws / gla_recurrent_bwd_ws: head dimension 256 (two passes of the D=128 matrix-core kernels,
+    their partial results in the caller's workspace), few long sequences (segments side by side: a dozen kernels
+    per call, the states between them in the workspace), and both at once."""
     from gla_jax_amd import _lib
     lib = _lib.load()
-    B, T, H, D = 2, 150, 2, 256
     dtype, dt = torch.bfloat16, _lib.GLA_BF16
     (h0n, gn, vn, kn, qn), (h0, g, v, k, q) = gpu_inputs(B, T, H, D, 3.0, seed=79, dtype=dtype)
     dhTn, doutn = cotangents(h0n, vn, 11, dtype)

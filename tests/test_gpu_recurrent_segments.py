@@ -1,0 +1,108 @@
+"""recurrent_gla on few sequences: with a workspace the C entry points run every sequence as S segments side by
+side (a pass from zero states, a scan over the segments, the real pass; the backward likewise for the states'
+cotangents).  Checked against the oracle like every other recurrent_gla case, and against the same call without a
+workspace (the sequences run whole): the two may differ by the order of fp32 sums only."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gla_oracle as O
+from tests.util import check_recurrent_outputs, cotangents, fmt_log, gpu_inputs, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+# dtype, B, T, H, D, reverse, gate shift: shapes at which gla_recurrent_*_workspace_bytes ask for segments
+CASES = [
+    (torch.bfloat16, 1, 1024, 2, 64, False, 3.0),
+    (torch.bfloat16, 1, 1024, 2, 64, True, 3.0),
+    (torch.bfloat16, 2, 2048, 1, 128, False, 5.0),
+    (torch.bfloat16, 1, 2048, 1, 128, True, 0.0),
+    (torch.float32, 1, 1024, 2, 32, False, 3.0),
+    (torch.float32, 1, 1024, 1, 64, True, 1.0),
+    (torch.bfloat16, 1, 1024, 3, 16, False, 3.0),
+    (torch.bfloat16, 2, 1024, 1, 256, False, 3.0),
+    (torch.bfloat16, 1, 1024, 1, 256, True, 3.0),
+    (torch.bfloat16, 1, 1280, 2, 64, False, 3.0),       # segments of 320 steps: not a multiple of the kernels' blocks
+    (torch.bfloat16, 1, 512, 2, 128, False, 3.0),       # two segments (bf16 at head dimensions 128 and 256 only)
+    (torch.bfloat16, 2, 512, 1, 128, True, 1.0),
+    (torch.bfloat16, 1, 512, 1, 256, False, 3.0),
+]
+
+
+def _sizes(B, T, H, D, dtype):
+    from gla_jax_amd import _lib
+    lib = _lib.load()
+    dt = _lib.GLA_BF16 if dtype == torch.bfloat16 else _lib.GLA_F32
+    return (lib.gla_recurrent_fwd_workspace_bytes(B, T, H, D, D, dt),
+            lib.gla_recurrent_bwd_workspace_bytes(B, T, H, D, D, dt))
+
+
+@pytest.mark.parametrize("dtype,B,T,H,D,reverse,shift", CASES)
+def test_segmented_recurrent_gla_matches_oracle(dtype, B, T, H, D, reverse, shift):
+    from gla_jax_amd import recurrent_gla
+    assert min(_sizes(B, T, H, D, dtype)) > 0, "the case is meant to run in segments"
+    (h0, g, v, k, q), dev = gpu_inputs(B, T, H, D, shift, seed=T + D, dtype=dtype)
+    g = g.copy()
+    g[:, 300::411] = -200.0                    # resets, one of them right behind a segment boundary or two
+    g[:, 255] = -30.0
+    dev[1] = to_dev(g, torch.float32)
+    dhT, dout = cotangents(h0, v, 5, dtype)
+    dev = [t.clone().requires_grad_(True) for t in dev]
+    hT, out = recurrent_gla(*dev, reverse=reverse)
+    loss = (hT.float() * to_dev(dhT, dtype).float()).sum() + (out.float() * to_dev(dout, dtype).float()).sum()
+    grads = torch.autograd.grad(loss, dev)
+    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=reverse)
+    print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads)))
+
+
+@pytest.mark.parametrize("dtype,B,T,H,D,reverse", [(torch.bfloat16, 1, 1024, 2, 64, False),
+                                                    (torch.bfloat16, 1, 1024, 1, 128, True),
+                                                    (torch.float32, 1, 1024, 2, 32, False)])
+def test_segments_agree_with_whole_sequences(dtype, B, T, H, D, reverse):
+    """The same call through gla_recurrent_fwd / _bwd (no workspace: whole sequences) and through the _ws entry
+    points (segments).  fp32 state hand-over, so the results differ by fp32 summation order: a rounding step of the
+    stored type at most on a few elements, far below the parity bound."""
+    from gla_jax_amd import _lib
+    lib = _lib.load()
+    dt = _lib.GLA_BF16 if dtype == torch.bfloat16 else _lib.GLA_F32
+    (h0n, gn, vn, kn, qn), (h0, g, v, k, q) = gpu_inputs(B, T, H, D, 3.0, seed=91, dtype=dtype)
+    dhTn, doutn = cotangents(h0n, vn, 12, dtype)
+    dhT, dout = to_dev(dhTn, dtype), to_dev(doutn, dtype)
+    p = lambda t: t.data_ptr()
+    u8 = lambda n: torch.empty(n, dtype=torch.uint8, device="cuda")
+    nf, nb = _sizes(B, T, H, D, dtype)
+    assert nf > 0 and nb > 0
+    ws_f, ws_b = u8(nf), u8(nb)
+    outs = lambda: [torch.empty_like(h0), torch.empty_like(v), torch.empty_like(h0), torch.empty_like(g),
+                    torch.empty_like(v), torch.empty_like(k), torch.empty_like(q)]
+    st = torch.cuda.current_stream().cuda_stream
+    rv = int(reverse)
+    whole, seg = outs(), outs()
+    hT, out, dh0, dg, dv, dk, dq = whole
+    _lib.check("gla_recurrent_fwd", lib.gla_recurrent_fwd(st, B, T, H, D, D, dt, dt, dt, rv, p(h0), p(g), p(v), p(k), p(q),
+                                                          p(hT), p(out)))
+    _lib.check("gla_recurrent_bwd", lib.gla_recurrent_bwd(st, B, T, H, D, D, dt, dt, dt, rv, p(h0), p(g), p(v), p(k), p(q),
+                                                          p(hT), p(dhT), p(dout), p(dh0), p(dg), p(dv), p(dk), p(dq)))
+    hT, out, dh0, dg, dv, dk, dq = seg
+    _lib.check("gla_recurrent_fwd_ws", lib.gla_recurrent_fwd_ws(st, B, T, H, D, D, dt, dt, dt, rv, p(h0), p(g), p(v), p(k),
+                                                                p(q), p(hT), p(out), p(ws_f), nf))
+    _lib.check("gla_recurrent_bwd_ws", lib.gla_recurrent_bwd_ws(st, B, T, H, D, D, dt, dt, dt, rv, p(h0), p(g), p(v), p(k),
+                                                                p(q), p(hT), p(dhT), p(dout), p(dh0), p(dg), p(dv), p(dk),
+                                                                p(dq), p(ws_b), nb))
+    torch.cuda.synchronize()
+    for name, a, b in zip(("hidden_final", "out", "dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), whole, seg):
+        a, b = to_np(a), to_np(b)
+        rms = float(np.sqrt(np.mean(a ** 2)))
+        worst = float(np.abs(a - b).max()) / rms
+        frac = float(np.mean(a != b))
+        print(f"{name}: max difference {worst:.2e} of an RMS, {100 * frac:.2f} % of the elements differ")
+        # bf16 results: one rounding step of a value of 8 RMS is 3.1e-2 RMS, on few elements.  d(log_fgate) (fp32)
+        # of bf16 data: the running sum over the later steps starts from sum_v d(state) * state at a segment's end
+        # where the whole sequence carries the sum of its terms, two forms whose own errors are 1e-4 each (as
+        # against the oracle).  fp32 data: summation order only.
+        if dtype == torch.float32:
+            assert worst <= 2e-5, name
+        elif name == "dlog_fgate":
+            assert worst <= 1e-3, name
+        else:
+            assert worst <= 4e-2 and frac <= 0.02, name
