@@ -562,8 +562,9 @@ struct TimeSplit {
     bool on() const { return S > 1; }
     // forward: entering states, the segments' own contributions, gate sums
     size_t fwd() const { return on() ? 2 * hid + sums : 0; }
-    // backward: the same and the entering cotangents
-    size_t bwd() const { return on() ? 3 * hid + sums : 0; }
+    // backward: the same, the cotangents that leave the segments, and a second array of contributions for an fp32
+    // dout beside bf16 data (two passes)
+    size_t bwd() const { return on() ? 4 * hid + sums : 0; }
 };
 static size_t inner_fwd_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int dtype)
 {
@@ -673,7 +674,7 @@ extern "C" int gla_recurrent_fwd_ws(void *stream, int64_t B, int64_t T, int64_t 
     e = recurrent_fwd_inner(stream, B * ts.S, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, entering, log_fgate,
                             value, key, query, loc, out, inner_ws, true);
     if (e) return e;
-    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, hidden_init, loc, sums, nullptr, 0,
+    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, hidden_init, loc, nullptr, sums, nullptr, 0,
                                  reverse, entering, hidden_final);
     if (e) return e;
     return recurrent_fwd_inner(stream, B * ts.S, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, entering,
@@ -792,16 +793,19 @@ extern "C" int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t 
     if (!workspace || workspace_bytes < need) return GLA_ERR_WORKSPACE;
     if (!gla::aligned16(workspace)) return GLA_ERR_ALIGN;
     const gla::TimeSplit ts(B, T, H, DK, dtype);
-    // The pass for the states' cotangents reads dout where the forward kernels read value, so dout must have value's
-    // type: with an fp32 dout beside bf16 data (the recurrent_gla_naive flavour) the sequences run whole.
-    if (!ts.on() || out_dtype != dtype)
+    // The pass for the states' cotangents reads dout where the forward kernels read value, so dout must come in
+    // value's type.  An fp32 dout beside bf16 data (the recurrent_gla_naive flavour) is cut into two bf16 arrays, head
+    // and remainder, whose passes' states add (the pass is linear in it); that needs the lean kernels, which write no
+    // `out`: where there are none (D = 16, 32) such a call runs the sequences whole.
+    const bool split_dout = out_dtype != dtype;
+    if (!ts.on() || (split_dout && DK < 64))
         return recurrent_bwd_inner(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
                                    log_fgate, value, key, query, hidden_final, dhidden_final, dout, dhidden_init,
                                    dlog_fgate, dvalue, dkey, dquery, DK == 256 ? (unsigned char *)workspace + ts.bwd() : nullptr);
     hipStream_t st = (hipStream_t)stream;
     unsigned char *ws = (unsigned char *)workspace;
     float *entering = (float *)ws, *loc = (float *)(ws + ts.hid), *dleaving = (float *)(ws + 2 * ts.hid),
-          *sums = (float *)(ws + 3 * ts.hid);
+          *loc_rem = (float *)(ws + 3 * ts.hid), *sums = (float *)(ws + 4 * ts.hid);
     void *inner_ws = DK == 256 ? ws + ts.bwd() : nullptr;      // sized for the backward, which needs more
     const int64_t BS = B * ts.S;
     // 1. the states that enter the segments, as the forward formed them; the pass's `out` lands in dquery, which the
@@ -813,8 +817,8 @@ extern "C" int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t 
     e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, entering, log_fgate, value,
                             key, query, loc, dquery, inner_ws, true);
     if (e) return e;
-    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, hidden_init, loc, sums, nullptr, 0, reverse,
-                                 entering, nullptr);
+    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, hidden_init, loc, nullptr, sums, nullptr, 0,
+                                 reverse, entering, nullptr);
     if (e) return e;
     // 2. the cotangents of the states that leave the segments.  d(state) obeys the state's recurrence against time
     //    with query for key and dout for value, the decay between two steps being the later step's gate: the same
@@ -824,13 +828,27 @@ extern "C" int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t 
     if (e) return e;
     e = gla::launch_zero_fill(st, dleaving, ts.hid);
     if (e) return e;
-    e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, !reverse, dleaving, dlog_fgate, dout,
-                            query, key, loc, dkey, inner_ws, true);
-    if (e) return e;
+    const float *loc2 = nullptr;
+    if (split_dout) {
+        // dkey and dvalue hold the two halves of dout until the backward proper writes its results there
+        e = gla::launch_head_remainder(st, B * T * H * DV, (const float *)dout, dkey, dvalue);
+        if (e) return e;
+        e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, dtype, !reverse, dleaving, dlog_fgate, dkey,
+                                query, key, loc, nullptr, inner_ws, true);
+        if (e) return e;
+        e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, dtype, !reverse, dleaving, dlog_fgate, dvalue,
+                                query, key, loc_rem, nullptr, inner_ws, true);
+        if (e) return e;
+        loc2 = loc_rem;
+    } else {
+        e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, !reverse, dleaving, dlog_fgate,
+                                dout, query, key, loc, dkey, inner_ws, true);
+        if (e) return e;
+    }
     // what enters segment p from the steps behind it: the gate of p's first step (in the order of the recurrence)
     // times its own contribution, plus its whole decay times what entered from further behind; after the last
     // segment that is dhidden_init
-    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, dhidden_final, loc, sums, log_fgate,
+    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, dhidden_final, loc, loc2, sums, log_fgate,
                                  reverse ? (int)ts.L - 1 : 0, !reverse, dleaving, dhidden_init);
     if (e) return e;
     // 3. the backward proper, every segment with its entering state and its leaving cotangent: the gate gradient's

@@ -54,11 +54,13 @@ __global__ __launch_bounds__(256) void shift_rows_kernel(const float *__restrict
 }
 
 // One thread per 4 neighbouring value features of a (b, h, dk) state row, a loop over the segments.
+// loc2 (may be null) is a second array of contributions, added to the first.
 __global__ __launch_bounds__(256) void segment_scan_kernel(const void *__restrict__ init, const float *__restrict__ loc,
-                                                           const float *__restrict__ sums, const float *__restrict__ g,
-                                                           float *__restrict__ entering, void *__restrict__ final,
-                                                           int64_t n4, int S, int L, int H, int D, int hdt, int edge_row,
-                                                           int descending)
+                                                           const float *__restrict__ loc2,
+                                                           const float *__restrict__ sums,
+                                                           const float *__restrict__ g, float *__restrict__ entering,
+                                                           void *__restrict__ final, int64_t n4, int S, int L, int H,
+                                                           int D, int hdt, int edge_row, int descending)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n4) return;
@@ -73,14 +75,32 @@ __global__ __launch_bounds__(256) void segment_scan_kernel(const void *__restric
         const int p = descending ? S - 1 - j : j;
         const int64_t seg = b * S + p;
         const int64_t o = (seg * H + h) * dd + in_state;
+        f32x4 l = *reinterpret_cast<const f32x4 *>(loc + o);
+        if (loc2) l += *reinterpret_cast<const f32x4 *>(loc2 + o);
         *reinterpret_cast<f32x4 *>(entering + o) = f32x4{x[0], x[1], x[2], x[3]};
-        const f32x4 l = *reinterpret_cast<const f32x4 *>(loc + o);
         const float a = expf(sums[(seg * H + h) * (int64_t)D + dk]);
         const float w = g ? expf(g[((seg * L + edge_row) * H + h) * (int64_t)D + dk]) : 1.f;
 #pragma unroll
         for (int c = 0; c < 4; ++c) x[c] = a * x[c] + w * l[c];
     }
     if (final) store_hidden<4>(final, hdt, e, x);
+}
+
+// hi = the bf16 nearest to x, lo = the bf16 nearest to what that leaves over; 8 elements per thread
+__global__ __launch_bounds__(256) void head_remainder_kernel(const float *__restrict__ x, __bf16 *__restrict__ hi,
+                                                             __bf16 *__restrict__ lo, int64_t n8)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    float a[8], h[8], l[8];
+    load_vec<float, 8>(x + i * 8, a);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        h[j] = (float)(__bf16)a[j];
+        l[j] = a[j] - h[j];
+    }
+    store_vec<__bf16, 8>(hi + i * 8, h);
+    store_vec<__bf16, 8>(lo + i * 8, l);
 }
 
 __global__ __launch_bounds__(256) void zero_fill_kernel(f32x4 *__restrict__ dst, int64_t n16)
@@ -123,13 +143,20 @@ int launch_shift_rows(hipStream_t st, int64_t B, int64_t T, int64_t row_len, con
 }
 
 int launch_segment_scan(hipStream_t st, int64_t B, int64_t S, int64_t L, int64_t H, int D, int hdt, const void *init,
-                        const float *loc, const float *sums, const float *g, int edge_row, int descending,
-                        float *entering, void *final)
+                        const float *loc, const float *loc2, const float *sums, const float *g, int edge_row,
+                        int descending, float *entering, void *final)
 {
     const int64_t n4 = B * H * D * D / 4;
     if (!grid_fits(n4) || S > 0x7fffffffLL || L > 0x7fffffffLL) return GLA_ERR_SHAPE;
-    hipLaunchKernelGGL(segment_scan_kernel, grid_for(n4), dim3(256), 0, st, init, loc, sums, g, entering, final, n4,
+    hipLaunchKernelGGL(segment_scan_kernel, grid_for(n4), dim3(256), 0, st, init, loc, loc2, sums, g, entering, final, n4,
                        (int)S, (int)L, (int)H, D, hdt, edge_row, descending);
+    return launch_status();
+}
+
+int launch_head_remainder(hipStream_t st, int64_t n, const float *x, void *hi, void *lo)
+{
+    if (n % 8 != 0 || !grid_fits(n / 8)) return GLA_ERR_SHAPE;
+    hipLaunchKernelGGL(head_remainder_kernel, grid_for(n / 8), dim3(256), 0, st, x, (__bf16 *)hi, (__bf16 *)lo, n / 8);
     return launch_status();
 }
 

@@ -13,12 +13,16 @@ int launch_segment_gate_sums(hipStream_t st, int64_t B, int64_t S, int64_t L, in
 // such neighbour.  Rows are [H*D] floats, T rows per batch entry.
 int launch_shift_rows(hipStream_t st, int64_t B, int64_t T, int64_t row_len, const float *src, float *dst, int dir);
 // The recurrence over segments, elementwise over a [D][D] state per (b, h):
-//     x <- exp(sums[b][p][h][dk]) * x + exp(edge) * loc[b][p][h][dk][dv],       p ascending, or descending from S-1,
+//     x <- exp(sums[b][p][h][dk]) * x + exp(edge) * (loc + loc2)[b][p][h][dk][dv],   p ascending, or descending from S-1,
 // with entering[b][p] = x before segment p's update (fp32) and `final` = x after the last one (type hdt; may be
-// null).  x starts as init[b][h] (type hdt).  edge = g[b][p*L + edge_row][h][dk] when g is given, else 0.
+// null).  x starts as init[b][h] (type hdt).  edge = g[b][p*L + edge_row][h][dk] when g is given, else 0.  loc2 may
+// be null.
 int launch_segment_scan(hipStream_t st, int64_t B, int64_t S, int64_t L, int64_t H, int D, int hdt, const void *init,
-                        const float *loc, const float *sums, const float *g, int edge_row, int descending,
-                        float *entering, void *final);
+                        const float *loc, const float *loc2, const float *sums, const float *g, int edge_row,
+                        int descending, float *entering, void *final);
+// hi[i] = bf16(x[i]), lo[i] = bf16(x[i] - hi[i]) for n floats (n a multiple of 8): a float array as two bf16 arrays
+// whose sum keeps 16 bits of mantissa
+int launch_head_remainder(hipStream_t st, int64_t n, const float *x, void *hi, void *lo);
 // n bytes of zeros (a multiple of 16, the address aligned to 16)
 int launch_zero_fill(hipStream_t st, void *dst, size_t n);
 

@@ -88,7 +88,7 @@ def test_chunk_plan_and_sizes():
     # recurrent_gla: a workspace at head dimension 256 (both passes' results in fp32 and the exchanged rows) and, at
     # every head dimension, where the sequences are few enough to run as S >= 4 segments of >= 256 steps side by
     # side (B*H*S <= 256 workgroups; S = 2 already for bf16 data at head dimensions 128 and 256): the segments'
-    # states in fp32, twice (backward: three times), and their gate sums
+    # states in fp32, twice (backward: four times), and their gate sums
     r256 = lambda x: (x + 255) & ~255
     for D in (16, 32, 64, 128):
         assert lib.gla_recurrent_fwd_workspace_bytes(16, 2048, 16, D, D, _lib.GLA_BF16) == 0    # 256 sequences
@@ -99,7 +99,7 @@ def test_chunk_plan_and_sizes():
         S = 8                                                                                   # 24 sequences of 4096 steps
         hid, sums = r256(B * S * H * D * D * 4), r256(B * S * H * D * 4)
         assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, D, D, _lib.GLA_BF16) == 2 * hid + sums
-        assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, D, D, _lib.GLA_F32) == 3 * hid + sums
+        assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, D, D, _lib.GLA_F32) == 4 * hid + sums
     assert lib.gla_recurrent_fwd_workspace_bytes(1, 1024, 64, 64, 64, _lib.GLA_BF16) == 2 * r256(4 * 64 * 64 * 64 * 4) + (
         r256(4 * 64 * 64 * 4))                                                                  # S = 4, the smallest
     rows32 = B * T * H * 256 * 4

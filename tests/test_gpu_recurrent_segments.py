@@ -106,3 +106,26 @@ def test_segments_agree_with_whole_sequences(dtype, B, T, H, D, reverse):
             assert worst <= 1e-3, name
         else:
             assert worst <= 4e-2 and frac <= 0.02, name
+
+
+@pytest.mark.parametrize("B,T,H,D,reverse", [(1, 1024, 2, 64, False), (1, 2048, 1, 128, True), (1, 1024, 1, 256, False),
+                                             (1, 1024, 2, 32, False)])
+def test_segmented_recurrent_gla_naive_flavour(B, T, H, D, reverse):
+    """bf16 data with an fp32 `out` and an fp32 cotangent for it (gla.py:37): the forward runs in segments like
+    recurrent_gla's; in the backward the pass for the states' cotangents takes dout as two bf16 arrays, head and
+    remainder, whose states add (D = 32 has no such pass and runs its backward on whole sequences)."""
+    from gla_jax_amd import recurrent_gla_naive
+    from tests.util import assert_plain
+    dtype = torch.bfloat16
+    assert min(_sizes(B, T, H, D, dtype)) > 0
+    (h0, g, v, k, q), dev = gpu_inputs(B, T, H, D, 3.0, seed=T + D + 1, dtype=dtype)
+    dhT, dout = cotangents(h0, v, 6, torch.float32)
+    dhT = O.bf16_round(dhT)
+    dev = [t.clone().requires_grad_(True) for t in dev]
+    hT, out = recurrent_gla_naive(*dev, reverse=reverse)
+    assert out.dtype == torch.float32 and hT.dtype == dtype
+    loss = (hT.float() * to_dev(dhT, dtype).float()).sum() + (out * to_dev(dout, torch.float32)).sum()
+    grads = torch.autograd.grad(loss, dev)
+    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=reverse)
+    assert_plain("out", to_np(out), exp[6], 1e-4)
+    print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads, out_fp32=True)))
