@@ -63,6 +63,8 @@ WORKLOADS = {
     "chunk": ("chunk", 4, 4096, 6, 128, 128, 5.0),       # BASELINE configs[1]/[2] (headline metric)
     "long": ("chunk", 1, 32768, 8, 128, 128, 0.0),       # BASELINE configs[3]
     "recurrent": ("recurrent", 16, 2048, 16, 64, 0, 3.0),  # BASELINE configs[4]
+    # the shape of the reference's own script (gla.py:1405-1410): 64 sequences, which run as 4 segments each
+    "recurrent_few": ("recurrent", 4, 4096, 16, 128, 0, 3.0),
     # the two scan operators of ops.py on their own, at the sizes chunk_gla gives them at the headline shape
     "scans": ("scans", 4, 4096, 6, 128, 128, 5.0),
 }
