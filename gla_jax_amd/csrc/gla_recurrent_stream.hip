@@ -107,8 +107,9 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             gN[ks] = ld8(g + rowN + 32 * ks + 8 * c);
-            qN[ks] = ld8(q + rowN + 32 * ks + 8 * c);
             kN[ks] = ld8(k + rowN + 32 * ks + 8 * c);
+            if constexpr (!STATE) qN[ks] = ld8(q + rowN + 32 * ks + 8 * c);
+            else qN[ks] = kN[ks];                             // nothing uses the query side of a lean pass
             vN[ks] = ld8(v + rowN + 32 * ks + 8 * c);
         }
     };
