@@ -34,7 +34,7 @@ template <> struct OutPack<float> {
 // sequence runs as segments side by side): the scores of earlier sub-blocks, the output products and the stores
 // of `out` are left out, and so is the copy of the state that those products read.
 template <typename TO, int C, int D, bool STATE = false>
-__global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
+__global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_kernel(
     const void *__restrict__ h0, const float *__restrict__ g, const __bf16 *__restrict__ v,
     const __bf16 *__restrict__ k, const __bf16 *__restrict__ q, void *__restrict__ hT,
     TO *__restrict__ out, int T_len, int H, int reverse, int hdt)
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(C * 4) void recurrent_stream_fwd_kernel(
     T *Kl = Kh + C * LS;                           // [C][LS]  what the bf16 rounding of Kh leaves over
     T *St = Kl + C * LS;                           // [D][LS]  state at the start of the block, [dv][dk]: bf16 head
     T *Sl = St + D * LS;                           // [D][LS]  ... and the bf16 of what the head leaves over
-    float *rtab = reinterpret_cast<float *>(Sl + D * LS);   // [NB][D] exp(tau_m)
+    float *rtab = reinterpret_cast<float *>(STATE ? St : Sl + D * LS);   // [NB][D] exp(tau_m)
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -261,7 +261,8 @@ static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, int 
 {
     typedef __bf16 T;
     constexpr int LS = TileGeom<T, D>::kStride;
-    const size_t lds = (size_t)(3 * C + 2 * D) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
+    // (the lean form has no copy of the state in LDS; its table of decays moves up to where that copy would start)
+    const size_t lds = (size_t)(3 * C + (STATE ? 0 : 2 * D)) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
     auto kern = recurrent_stream_fwd_kernel<TO, C, D, STATE>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
