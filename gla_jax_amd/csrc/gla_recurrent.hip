@@ -543,9 +543,13 @@ extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, 
 namespace gla {
 constexpr int64_t kComputeUnits = 256;       // MI355X
 constexpr int64_t kMinSegment = 256;         // steps: below this the extra pass costs more than the idle units
+// bf16 data at head dimensions 64, 128 (and 256 as two passes of 128): the forward kernel has a form that leaves out
+// everything but the state
+static inline bool has_lean_pass(int dtype, int64_t DK) { return dtype == GLA_BF16 && DK >= 64; }
 struct TimeSplit {
     int64_t S = 1, L = 0;
-    size_t hid = 0, sums = 0;
+    int64_t F = 1, Lf = 0;       // the lean passes run every segment as F pieces of Lf steps
+    size_t hid = 0, hidf = 0, sums = 0;
     TimeSplit(int64_t B, int64_t T, int64_t H, int64_t DK, int dtype)
     {
         const int64_t seqs = B * H * (DK == 256 ? 2 : 1);    // head dimension 256 runs as 2H heads of 128
@@ -554,17 +558,25 @@ struct TimeSplit {
         // Two segments mean two passes over half the steps each: that pays only where the first pass is the lean one
         // (bf16 data) and the kernels are heavy (128 features: 1.47 -> 1.32 ms at B16 T2048 H8; 64 features:
         // 0.43 -> 0.45 ms).  From four segments on it pays everywhere.
-        if (S < (dtype == GLA_BF16 && DK >= 128 ? 2 : 4)) S = 1;
+        const bool heavy = dtype == GLA_BF16 && DK >= 128;
+        if (S < (heavy ? 2 : 4)) S = 1;
         L = T / S;
+        // The lean kernel of 128 features fits a compute unit twice (256 registers, 52 KB of LDS) where the full
+        // kernels fit once: its passes take every segment in two pieces (512 workgroups: 100 -> 70 us at 1024 steps
+        // per segment), and the scan puts the pieces together.  Pieces of 128 steps are two iterations of the kernel
+        // and lose what the second workgroup gains.
+        if (S > 1 && heavy && L % 2 == 0 && L / 2 >= kMinSegment && B * S * 2 <= 65535) F = 2;
+        Lf = L / F;
         hid = SplitSizes::round_up256((size_t)B * S * H * DK * DK * 4);
-        sums = SplitSizes::round_up256((size_t)B * S * H * DK * 4);
+        hidf = SplitSizes::round_up256((size_t)B * S * F * H * DK * DK * 4);
+        sums = SplitSizes::round_up256((size_t)B * S * F * H * DK * 4);
     }
     bool on() const { return S > 1; }
-    // forward: entering states, the segments' own contributions, gate sums
-    size_t fwd() const { return on() ? 2 * hid + sums : 0; }
+    // forward: entering states, the pieces' own contributions, gate sums
+    size_t fwd() const { return on() ? hid + hidf + sums : 0; }
     // backward: the same, the cotangents that leave the segments, and a second array of contributions for an fp32
     // dout beside bf16 data (two passes)
-    size_t bwd() const { return on() ? 4 * hid + sums : 0; }
+    size_t bwd() const { return on() ? 2 * hid + 2 * hidf + sums : 0; }
 };
 static size_t inner_fwd_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int dtype)
 {
@@ -581,7 +593,7 @@ extern "C" size_t gla_recurrent_fwd_workspace_bytes(int64_t B, int64_t T, int64_
 {
     if (gla::check_recurrent(B, T, H, DK, DV, dtype, GLA_F32, GLA_F32) || 2 * H > 65535) return 0;
     const gla::TimeSplit ts(B, T, H, DK, dtype);      // the passes run on B*S batch entries of L steps: their state blocks count
-    return ts.fwd() + gla::inner_fwd_bytes(B * ts.S, ts.L, H, DK, dtype);
+    return ts.fwd() + gla::inner_fwd_bytes(B * ts.S * ts.F, ts.Lf, H, DK, dtype);
 }
 
 extern "C" size_t gla_recurrent_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV,
@@ -589,7 +601,7 @@ extern "C" size_t gla_recurrent_bwd_workspace_bytes(int64_t B, int64_t T, int64_
 {
     if (gla::check_recurrent(B, T, H, DK, DV, dtype, GLA_F32, GLA_F32) || 2 * H > 65535) return 0;
     const gla::TimeSplit ts(B, T, H, DK, dtype);
-    return ts.bwd() + gla::inner_bwd_bytes(B * ts.S, ts.L, H, DK, dtype);
+    return ts.bwd() + gla::inner_bwd_bytes(B * ts.S * ts.F, ts.Lf, H, DK, dtype);
 }
 
 // One pass over whole sequences; arguments checked by the caller.  Head dimension 256 with a workspace: two passes
@@ -600,7 +612,8 @@ static int recurrent_fwd_inner(void *stream, int64_t B, int64_t T, int64_t H, in
                                void *hidden_final, void *out, void *workspace, bool state_only = false)
 {
     // state_only: the caller wants hidden_final alone and `out` is a buffer it will overwrite.  The matrix-core
-    // kernels have a form without the output products; the other kernels write the unused `out`.
+    // kernels have a form without the output products (hidden_init may be null there: zeros); the other kernels
+    // write the unused `out`.
     const bool lean = state_only && dtype == GLA_BF16;
     if (lean && (DK == 64 || DK == 128))
         return gla::launch_recurrent_stream_state((hipStream_t)stream, B, T, H, DK, reverse, hidden_dtype, hidden_init,
@@ -613,18 +626,21 @@ static int recurrent_fwd_inner(void *stream, int64_t B, int64_t T, int64_t H, in
     unsigned char *ws = (unsigned char *)workspace;
     unsigned char *v_sw = ws, *out1 = v_sw + z.rows_e, *out2 = out1 + z.rows_f32, *h0_same = out2 + z.rows_f32,
                   *h0_cross = h0_same + z.hid, *hT_same = h0_cross + z.hid, *hT_cross = hT_same + z.hid;
-    int e = gla::launch_hidden_blocks(st, hidden_dtype, B * H, const_cast<void *>(hidden_init), h0_same, h0_cross, 1);
-    if (e) return e;
+    int e = 0;
+    if (hidden_init) {      // (a lean pass may start from zeros: no initial state given)
+        e = gla::launch_hidden_blocks(st, hidden_dtype, B * H, const_cast<void *>(hidden_init), h0_same, h0_cross, 1);
+        if (e) return e;
+    }
     e = gla::launch_swap_halves(st, dtype, B * T * H, v_sw, value);
     if (e) return e;
     // key half a with value half a on the arrays as they lie, then key half a with the other value half; `out` of
     // both in fp32 (the recurrent_gla_naive flavour of the 128-feature kernels)
     if (lean) {
-        e = gla::launch_recurrent_stream_state(st, B, T, 2 * H, 128, reverse, hidden_dtype, h0_same, log_fgate, value, key,
-                                               query, hT_same);
+        e = gla::launch_recurrent_stream_state(st, B, T, 2 * H, 128, reverse, hidden_dtype, hidden_init ? h0_same : nullptr,
+                                               log_fgate, value, key, query, hT_same);
         if (e) return e;
-        e = gla::launch_recurrent_stream_state(st, B, T, 2 * H, 128, reverse, hidden_dtype, h0_cross, log_fgate, v_sw, key,
-                                               query, hT_cross);
+        e = gla::launch_recurrent_stream_state(st, B, T, 2 * H, 128, reverse, hidden_dtype,
+                                               hidden_init ? h0_cross : nullptr, log_fgate, v_sw, key, query, hT_cross);
         if (e) return e;
         return gla::launch_hidden_blocks(st, hidden_dtype, B * H, hidden_final, hT_same, hT_cross, 0);
     }
@@ -664,18 +680,23 @@ extern "C" int gla_recurrent_fwd_ws(void *stream, int64_t B, int64_t T, int64_t 
                                    log_fgate, value, key, query, hidden_final, out, workspace);
     hipStream_t st = (hipStream_t)stream;
     unsigned char *ws = (unsigned char *)workspace;
-    float *entering = (float *)ws, *loc = (float *)(ws + ts.hid), *sums = (float *)(ws + 2 * ts.hid);
+    float *entering = (float *)ws, *loc = (float *)(ws + ts.hid), *sums = (float *)(ws + ts.hid + ts.hidf);
     void *inner_ws = DK == 256 ? ws + ts.fwd() : nullptr;
-    int e = gla::launch_zero_fill(st, entering, ts.hid);
+    const bool lean = gla::has_lean_pass(dtype, DK);
+    const int64_t pieces = B * ts.S * ts.F;
+    int e = gla::launch_segment_gate_sums(st, B, ts.S * ts.F, ts.Lf, H, (int)DK, log_fgate, sums);
     if (e) return e;
-    e = gla::launch_segment_gate_sums(st, B, ts.S, ts.L, H, (int)DK, log_fgate, sums);
+    if (!lean) {            // (F = 1 then) the full kernels want an initial state: zeros
+        e = gla::launch_zero_fill(st, entering, ts.hid);
+        if (e) return e;
+    }
+    // every piece from a zero state: its own contribution to the state that leaves it (where this is a full pass, it
+    // writes an `out` that the pass below writes again)
+    e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, lean ? nullptr : entering,
+                            log_fgate, value, key, query, loc, out, inner_ws, true);
     if (e) return e;
-    // every segment from a zero state: its own contribution to the state that leaves it (`out` is written again below)
-    e = recurrent_fwd_inner(stream, B * ts.S, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, entering, log_fgate,
-                            value, key, query, loc, out, inner_ws, true);
-    if (e) return e;
-    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, hidden_init, loc, nullptr, sums, nullptr, 0,
-                                 reverse, entering, hidden_final);
+    e = gla::launch_segment_scan(st, B, ts.S, ts.F, ts.Lf, H, (int)DK, hidden_dtype, hidden_init, loc, nullptr, sums,
+                                 nullptr, 0, reverse, entering, hidden_final);
     if (e) return e;
     return recurrent_fwd_inner(stream, B * ts.S, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, entering,
                                log_fgate, value, key, query, loc, out, inner_ws);
@@ -804,52 +825,55 @@ extern "C" int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t 
                                    dlog_fgate, dvalue, dkey, dquery, DK == 256 ? (unsigned char *)workspace + ts.bwd() : nullptr);
     hipStream_t st = (hipStream_t)stream;
     unsigned char *ws = (unsigned char *)workspace;
-    float *entering = (float *)ws, *loc = (float *)(ws + ts.hid), *dleaving = (float *)(ws + 2 * ts.hid),
-          *loc_rem = (float *)(ws + 3 * ts.hid), *sums = (float *)(ws + 4 * ts.hid);
+    float *entering = (float *)ws, *dleaving = (float *)(ws + ts.hid), *loc = (float *)(ws + 2 * ts.hid),
+          *loc_rem = (float *)(ws + 2 * ts.hid + ts.hidf), *sums = (float *)(ws + 2 * ts.hid + 2 * ts.hidf);
     void *inner_ws = DK == 256 ? ws + ts.bwd() : nullptr;      // sized for the backward, which needs more
-    const int64_t BS = B * ts.S;
-    // 1. the states that enter the segments, as the forward formed them; the pass's `out` lands in dquery, which the
-    //    backward proper overwrites
-    int e = gla::launch_zero_fill(st, entering, ts.hid);
+    const int64_t BS = B * ts.S, pieces = BS * ts.F;
+    const bool lean = gla::has_lean_pass(dtype, DK);
+    // 1. the states that enter the segments, as the forward formed them (where the pass is a full one, its `out` lands
+    //    in dquery, which the backward proper overwrites)
+    int e = gla::launch_segment_gate_sums(st, B, ts.S * ts.F, ts.Lf, H, (int)DK, log_fgate, sums);
     if (e) return e;
-    e = gla::launch_segment_gate_sums(st, B, ts.S, ts.L, H, (int)DK, log_fgate, sums);
+    if (!lean) {
+        e = gla::launch_zero_fill(st, entering, ts.hid);
+        if (e) return e;
+        e = gla::launch_zero_fill(st, dleaving, ts.hid);
+        if (e) return e;
+    }
+    e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, lean ? nullptr : entering,
+                            log_fgate, value, key, query, loc, dquery, inner_ws, true);
     if (e) return e;
-    e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, entering, log_fgate, value,
-                            key, query, loc, dquery, inner_ws, true);
-    if (e) return e;
-    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, hidden_init, loc, nullptr, sums, nullptr, 0,
-                                 reverse, entering, nullptr);
+    e = gla::launch_segment_scan(st, B, ts.S, ts.F, ts.Lf, H, (int)DK, hidden_dtype, hidden_init, loc, nullptr, sums,
+                                 nullptr, 0, reverse, entering, nullptr);
     if (e) return e;
     // 2. the cotangents of the states that leave the segments.  d(state) obeys the state's recurrence against time
     //    with query for key and dout for value, the decay between two steps being the later step's gate: the same
     //    forward kernels in the other direction on the gates moved by one row (kept in dlog_fgate until the
-    //    backward proper writes there; the pass's `out` lands in dkey).
+    //    backward proper writes there; a full pass's `out` lands in dkey).
     e = gla::launch_shift_rows(st, B, T, H * DK, log_fgate, dlog_fgate, reverse ? -1 : 1);
-    if (e) return e;
-    e = gla::launch_zero_fill(st, dleaving, ts.hid);
     if (e) return e;
     const float *loc2 = nullptr;
     if (split_dout) {
         // dkey and dvalue hold the two halves of dout until the backward proper writes its results there
         e = gla::launch_head_remainder(st, B * T * H * DV, (const float *)dout, dkey, dvalue);
         if (e) return e;
-        e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, dtype, !reverse, dleaving, dlog_fgate, dkey,
+        e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, dtype, !reverse, nullptr, dlog_fgate, dkey,
                                 query, key, loc, nullptr, inner_ws, true);
         if (e) return e;
-        e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, dtype, !reverse, dleaving, dlog_fgate, dvalue,
-                                query, key, loc_rem, nullptr, inner_ws, true);
+        e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, dtype, !reverse, nullptr, dlog_fgate,
+                                dvalue, query, key, loc_rem, nullptr, inner_ws, true);
         if (e) return e;
         loc2 = loc_rem;
     } else {
-        e = recurrent_fwd_inner(stream, BS, ts.L, H, DK, DV, dtype, GLA_F32, out_dtype, !reverse, dleaving, dlog_fgate,
-                                dout, query, key, loc, dkey, inner_ws, true);
+        e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, out_dtype, !reverse,
+                                lean ? nullptr : dleaving, dlog_fgate, dout, query, key, loc, dkey, inner_ws, true);
         if (e) return e;
     }
-    // what enters segment p from the steps behind it: the gate of p's first step (in the order of the recurrence)
-    // times its own contribution, plus its whole decay times what entered from further behind; after the last
-    // segment that is dhidden_init
-    e = gla::launch_segment_scan(st, B, ts.S, ts.L, H, (int)DK, hidden_dtype, dhidden_final, loc, loc2, sums, log_fgate,
-                                 reverse ? (int)ts.L - 1 : 0, !reverse, dleaving, dhidden_init);
+    // what enters segment p from the steps behind it: per piece, the gate of its first step (in the order of the
+    // recurrence) times its own contribution, plus its whole decay times what entered from further behind; after
+    // the last piece that is dhidden_init
+    e = gla::launch_segment_scan(st, B, ts.S, ts.F, ts.Lf, H, (int)DK, hidden_dtype, dhidden_final, loc, loc2, sums,
+                                 log_fgate, reverse ? (int)ts.Lf - 1 : 0, !reverse, dleaving, dhidden_init);
     if (e) return e;
     // 3. the backward proper, every segment with its entering state and its leaving cotangent: the gate gradient's
     //    running sum starts from sum_v d(state) * state at the segment's end, which is what the steps behind it add

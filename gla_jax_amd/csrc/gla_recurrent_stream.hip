@@ -76,8 +76,8 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
     for (int i = 0; i < RT; ++i)
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
-            float t4[4];
-            load_hidden<4>(h0, hdt, bh * D * D + (int64_t)(16 * (nt0 + nt) + r) * D + 16 * (wv + i * NDV) + 4 * c, t4);
+            float t4[4] = {0.f, 0.f, 0.f, 0.f};     // no initial state given: zeros (the lean pass of a segment)
+            if (h0) load_hidden<4>(h0, hdt, bh * D * D + (int64_t)(16 * (nt0 + nt) + r) * D + 16 * (wv + i * NDV) + 4 * c, t4);
             S[i][nt] = f32x4{t4[0], t4[1], t4[2], t4[3]};
         }
     auto publish_state = [&]() {

@@ -13,6 +13,7 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
                                 void *hT, void *out);
 
 // The forward without its outputs: hidden_final alone (what a segment contributes to the state that leaves it).
+// h0 may be null: the state starts from zeros.
 int launch_recurrent_stream_state(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, const void *h0,
                                  const float *g, const void *v, const void *k, const void *q, void *hT);
 

@@ -64,14 +64,16 @@ __global__ __launch_bounds__(256) void shift_rows_kernel(const float *__restrict
     *reinterpret_cast<f32x4 *>(dst + i * 4) = x;
 }
 
-// One thread per 4 neighbouring value features of a (b, h, dk) state row, a loop over the segments.
+// One thread per 4 neighbouring value features of a (b, h, dk) state row, a loop over the segments.  The
+// contributions may come in pieces: every segment as F consecutive pieces of Lf steps each (S*F pieces per batch
+// entry, loc / loc2 / sums indexed by piece); `entering` is stored per segment, before its first piece.
 // loc2 (may be null) is a second array of contributions, added to the first.
 __global__ __launch_bounds__(256) void segment_scan_kernel(const void *__restrict__ init, const float *__restrict__ loc,
                                                            const float *__restrict__ loc2,
                                                            const float *__restrict__ sums,
                                                            const float *__restrict__ g, float *__restrict__ entering,
-                                                           void *__restrict__ final, int64_t n4, int S, int L, int H,
-                                                           int D, int hdt, int edge_row, int descending)
+                                                           void *__restrict__ final, int64_t n4, int S, int F, int Lf,
+                                                           int H, int D, int hdt, int edge_row, int descending)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n4) return;
@@ -80,17 +82,19 @@ __global__ __launch_bounds__(256) void segment_scan_kernel(const void *__restric
     const int64_t b = e / (dd * H);
     const int h = (int)(e / dd % H), dk = (int)(e / D % D);
     const int64_t in_state = e % dd;
+    const int P = S * F;
     float x[4];
     load_hidden<4>(init, hdt, e, x);
-    for (int j = 0; j < S; ++j) {
-        const int p = descending ? S - 1 - j : j;
-        const int64_t seg = b * S + p;
-        const int64_t o = (seg * H + h) * dd + in_state;
+    for (int j = 0; j < P; ++j) {
+        const int pf = descending ? P - 1 - j : j;      // the piece, in the order the recurrence meets them
+        const int64_t piece = b * P + pf;
+        const int64_t o = (piece * H + h) * dd + in_state;
         f32x4 l = *reinterpret_cast<const f32x4 *>(loc + o);
         if (loc2) l += *reinterpret_cast<const f32x4 *>(loc2 + o);
-        *reinterpret_cast<f32x4 *>(entering + o) = f32x4{x[0], x[1], x[2], x[3]};
-        const float a = expf(sums[(seg * H + h) * (int64_t)D + dk]);
-        const float w = g ? expf(g[((seg * L + edge_row) * H + h) * (int64_t)D + dk]) : 1.f;
+        if (j % F == 0)
+            *reinterpret_cast<f32x4 *>(entering + (((b * S + pf / F) * H + h) * dd + in_state)) = f32x4{x[0], x[1], x[2], x[3]};
+        const float a = expf(sums[(piece * H + h) * (int64_t)D + dk]);
+        const float w = g ? expf(g[((piece * Lf + edge_row) * H + h) * (int64_t)D + dk]) : 1.f;
 #pragma unroll
         for (int c = 0; c < 4; ++c) x[c] = a * x[c] + w * l[c];
     }
@@ -153,14 +157,14 @@ int launch_shift_rows(hipStream_t st, int64_t B, int64_t T, int64_t row_len, con
     return launch_status();
 }
 
-int launch_segment_scan(hipStream_t st, int64_t B, int64_t S, int64_t L, int64_t H, int D, int hdt, const void *init,
-                        const float *loc, const float *loc2, const float *sums, const float *g, int edge_row,
-                        int descending, float *entering, void *final)
+int launch_segment_scan(hipStream_t st, int64_t B, int64_t S, int64_t F, int64_t Lf, int64_t H, int D, int hdt,
+                        const void *init, const float *loc, const float *loc2, const float *sums, const float *g,
+                        int edge_row, int descending, float *entering, void *final)
 {
     const int64_t n4 = B * H * D * D / 4;
-    if (!grid_fits(n4) || S > 0x7fffffffLL || L > 0x7fffffffLL) return GLA_ERR_SHAPE;
+    if (!grid_fits(n4) || S * F > 0x7fffffffLL || Lf > 0x7fffffffLL || F < 1) return GLA_ERR_SHAPE;
     hipLaunchKernelGGL(segment_scan_kernel, grid_for(n4), dim3(256), 0, st, init, loc, loc2, sums, g, entering, final, n4,
-                       (int)S, (int)L, (int)H, D, hdt, edge_row, descending);
+                       (int)S, (int)F, (int)Lf, (int)H, D, hdt, edge_row, descending);
     return launch_status();
 }
 

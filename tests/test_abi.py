@@ -94,11 +94,15 @@ def test_chunk_plan_and_sizes():
         assert lib.gla_recurrent_fwd_workspace_bytes(16, 2048, 16, D, D, _lib.GLA_BF16) == 0    # 256 sequences
         assert lib.gla_recurrent_bwd_workspace_bytes(16, 2048, 8, D, D, _lib.GLA_F32) == 0      # 128: S would be 2
         assert lib.gla_recurrent_fwd_workspace_bytes(1, 500, 2, D, D, _lib.GLA_BF16) == 0       # segments below 256 steps
+        # (bf16 data at head dimension 128: the first pass takes every segment in F = 2 pieces, so its array of
+        # contributions and the gate sums count twice)
+        F = 2 if D == 128 else 1
         two = lib.gla_recurrent_fwd_workspace_bytes(16, 2048, 8, D, D, _lib.GLA_BF16)           # 128 sequences: S = 2
-        assert two == (2 * r256(16 * 2 * 8 * D * D * 4) + r256(16 * 2 * 8 * D * 4) if D == 128 else 0)
+        assert two == (3 * r256(16 * 2 * 8 * D * D * 4) + r256(16 * 4 * 8 * D * 4) if D == 128 else 0)
         S = 8                                                                                   # 24 sequences of 4096 steps
         hid, sums = r256(B * S * H * D * D * 4), r256(B * S * H * D * 4)
-        assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, D, D, _lib.GLA_BF16) == 2 * hid + sums
+        assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, D, D, _lib.GLA_BF16) == (1 + F) * hid + F * sums
+        assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, D, D, _lib.GLA_BF16) == (2 + 2 * F) * hid + F * sums
         assert lib.gla_recurrent_bwd_workspace_bytes(B, T, H, D, D, _lib.GLA_F32) == 4 * hid + sums
     assert lib.gla_recurrent_fwd_workspace_bytes(1, 1024, 64, 64, 64, _lib.GLA_BF16) == 2 * r256(4 * 64 * 64 * 64 * 4) + (
         r256(4 * 64 * 64 * 4))                                                                  # S = 4, the smallest

@@ -26,6 +26,8 @@ CASES = [
     (torch.bfloat16, 1, 512, 2, 128, False, 3.0),       # two segments (bf16 at head dimensions 128 and 256 only)
     (torch.bfloat16, 2, 512, 1, 128, True, 1.0),
     (torch.bfloat16, 1, 512, 1, 256, False, 3.0),
+    (torch.bfloat16, 1, 2048, 64, 128, False, 3.0),     # 4 segments of 512 steps, the lean passes in pieces of 256
+    (torch.bfloat16, 2, 2048, 16, 256, True, 3.0),
 ]
 
 
@@ -51,7 +53,14 @@ def test_segmented_recurrent_gla_matches_oracle(dtype, B, T, H, D, reverse, shif
     hT, out = recurrent_gla(*dev, reverse=reverse)
     loss = (hT.float() * to_dev(dhT, dtype).float()).sum() + (out.float() * to_dev(dout, dtype).float()).sum()
     grads = torch.autograd.grad(loss, dev)
-    exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=reverse)
+    if B * H >= 32:         # many sequences: the C restatement on all host threads (fp64); it walks forward in time,
+        from oracle import naive_c                     # and the reversed scan is that of the flipped sequence
+        fl = (lambda a: np.ascontiguousarray(a[:, ::-1])) if reverse else (lambda a: a)
+        dh0_, dg_, dv_, dk_, dq_, hT_, out_ = naive_c.naive_bwd(h0, fl(g), fl(v), fl(k), fl(q), dhT, fl(dout),
+                                                                dtype=np.float64, nthreads=16)
+        exp = (dh0_, fl(dg_), fl(dv_), fl(dk_), fl(dq_), hT_, fl(out_))
+    else:
+        exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=reverse)
     print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads)))
 
 
