@@ -271,7 +271,8 @@ class _RecurrentGLA(torch.autograd.Function):
         odt = _lib.GLA_F32 if out_fp32 else dt
         hT = torch.empty_like(h0)
         out = torch.empty(v.shape, dtype=torch.float32 if out_fp32 else v.dtype, device=v.device)
-        # a workspace is needed at head dimension 256 only (two passes of the 128-feature kernels)
+        # a workspace where the library can use one: head dimension 256 (two passes of the 128-feature kernels) and
+        # few long sequences (each runs as segments side by side); zero bytes elsewhere
         ws_bytes = lib.gla_recurrent_fwd_workspace_bytes(B, T, H, DK, DV, dt)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=v.device) if ws_bytes else None
         rc = lib.gla_recurrent_fwd_ws(_stream(), B, T, H, DK, DV, dt, _DT[h0.dtype], odt, int(bool(reverse)), _ptr(h0),

@@ -128,7 +128,8 @@ def recurrent_gla_forward_backward(hidden_init, log_fgate, value, key, query, re
 
 
 def _rec_workspace(key, value, which):
-    """The workspace of a recurrent_gla call as a byte array (head dimension 256 needs one, elsewhere 16 bytes)."""
+    """The workspace of a recurrent_gla call as a byte array (head dimension 256 and calls with few long sequences
+    use one; elsewhere 16 bytes that nobody reads)."""
     *lead, T, H, DK = key.shape
     B = 1
     for s in lead:

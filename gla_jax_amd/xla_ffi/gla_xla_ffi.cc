@@ -109,7 +109,7 @@ ffi::Error ChunkBwd(hipStream_t stream, int64_t chunk_size, ffi::Buffer<ffi::F32
 // forward rule, recurrent_gla_forward (gla.py:99-170); `reverse` as in gla.py:421-438.  The element type of
 // `out` selects the flavour: the value dtype for recurrent_gla, F32 for recurrent_gla_naive (gla.py:37).  The last
 // result is a workspace XLA allocates for the call, sized by gla_recurrent_fwd_workspace_bytes on the Python side
-// (head dimension 256 needs one; elsewhere it is a few bytes that nobody reads).
+// (head dimension 256 and calls with few long sequences use one; elsewhere it is a few bytes that nobody reads).
 ffi::Error RecurrentFwd(hipStream_t stream, bool reverse, ffi::AnyBuffer h0, ffi::Buffer<ffi::F32> g,
                         ffi::AnyBuffer v, ffi::AnyBuffer k, ffi::AnyBuffer q, ffi::Result<ffi::AnyBuffer> hT,
                         ffi::Result<ffi::AnyBuffer> out, ffi::Result<ffi::AnyBuffer> workspace)
