@@ -132,6 +132,10 @@ def test_entry_points_reject_bad_arguments_without_touching_the_gpu():
     assert rec(48, None, 0) == -2
     assert rec(256, None, 0) == -5
     assert rec(256, a, 64) == -5
+    # ... and where few long sequences run as segments (one sequence of 1024 steps: four segments)
+    seg = lambda ws, n: lib.gla_recurrent_fwd_ws(None, 1, 1024, 1, 64, 64, 1, 1, 1, 0, a, a, a, a, a, a, a, ws, n)
+    assert lib.gla_recurrent_fwd_workspace_bytes(1, 1024, 1, 64, 64, 1) > 64
+    assert seg(None, 0) == -5 and seg(a, 64) == -5 and seg(a + 4, 1 << 30) == -6
     assert lib.gla_recurrent_bwd_ws(None, 1, 8, 1, 256, 256, 1, 1, 1, 0, a, a, a, a, a, a, a, a, a, a, a, a, a,
                                     a, 64) == -5
     assert lib.gla_recurrent_bwd_ws(None, 1, 8, 1, 256, 256, 1, 1, 1, 0, a, a, a, a, a, a, a, a, a, a, a, a, None,
