@@ -609,15 +609,18 @@ extern "C" size_t gla_recurrent_bwd_workspace_bytes(int64_t B, int64_t T, int64_
 static int recurrent_fwd_inner(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK, int64_t DV, gla_dtype dtype,
                                gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse, const void *hidden_init,
                                const float *log_fgate, const void *value, const void *key, const void *query,
-                               void *hidden_final, void *out, void *workspace, bool state_only = false)
+                               void *hidden_final, void *out, void *workspace, bool state_only = false,
+                               int g_shift = 0)
 {
     // state_only: the caller wants hidden_final alone and `out` is a buffer it will overwrite.  The matrix-core
     // kernels have a form without the output products (hidden_init may be null there: zeros); the other kernels
     // write the unused `out`.
+    // g_shift (lean passes only): the gates are taken one row further on (+1) or back (-1), see the launcher.
     const bool lean = state_only && dtype == GLA_BF16;
+    if (g_shift && !(lean && DK >= 64)) return GLA_ERR_UNSUPPORTED;
     if (lean && (DK == 64 || DK == 128))
         return gla::launch_recurrent_stream_state((hipStream_t)stream, B, T, H, DK, reverse, hidden_dtype, hidden_init,
-                                                  log_fgate, value, key, query, hidden_final);
+                                                  log_fgate, value, key, query, hidden_final, g_shift);
     if (DK != 256 || !workspace)
         return recurrent_fwd_run(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
                                  log_fgate, value, key, query, hidden_final, out);
@@ -637,10 +640,11 @@ static int recurrent_fwd_inner(void *stream, int64_t B, int64_t T, int64_t H, in
     // both in fp32 (the recurrent_gla_naive flavour of the 128-feature kernels)
     if (lean) {
         e = gla::launch_recurrent_stream_state(st, B, T, 2 * H, 128, reverse, hidden_dtype, hidden_init ? h0_same : nullptr,
-                                               log_fgate, value, key, query, hT_same);
+                                               log_fgate, value, key, query, hT_same, g_shift);
         if (e) return e;
         e = gla::launch_recurrent_stream_state(st, B, T, 2 * H, 128, reverse, hidden_dtype,
-                                               hidden_init ? h0_cross : nullptr, log_fgate, v_sw, key, query, hT_cross);
+                                               hidden_init ? h0_cross : nullptr, log_fgate, v_sw, key, query, hT_cross,
+                                               g_shift);
         if (e) return e;
         return gla::launch_hidden_blocks(st, hidden_dtype, B * H, hidden_final, hT_same, hT_cross, 0);
     }
@@ -848,25 +852,32 @@ extern "C" int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t 
     if (e) return e;
     // 2. the cotangents of the states that leave the segments.  d(state) obeys the state's recurrence against time
     //    with query for key and dout for value, the decay between two steps being the later step's gate: the same
-    //    forward kernels in the other direction on the gates moved by one row (kept in dlog_fgate until the
-    //    backward proper writes there; a full pass's `out` lands in dkey).
-    e = gla::launch_shift_rows(st, B, T, H * DK, log_fgate, dlog_fgate, reverse ? -1 : 1);
-    if (e) return e;
+    //    forward kernels in the other direction with the gates taken one row further on.  The lean kernels read
+    //    them there; for the others a copy moved by one row is kept in dlog_fgate until the backward proper writes
+    //    there (and the pass's `out` lands in dkey).
+    const int shift = reverse ? -1 : 1;
+    const float *gates = log_fgate;
+    if (!lean) {
+        e = gla::launch_shift_rows(st, B, T, H * DK, log_fgate, dlog_fgate, shift);
+        if (e) return e;
+        gates = dlog_fgate;
+    }
+    const int gs = lean ? shift : 0;
     const float *loc2 = nullptr;
     if (split_dout) {
         // dkey and dvalue hold the two halves of dout until the backward proper writes its results there
         e = gla::launch_head_remainder(st, B * T * H * DV, (const float *)dout, dkey, dvalue);
         if (e) return e;
-        e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, dtype, !reverse, nullptr, dlog_fgate, dkey,
-                                query, key, loc, nullptr, inner_ws, true);
+        e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, dtype, !reverse, nullptr, gates, dkey,
+                                query, key, loc, nullptr, inner_ws, true, gs);
         if (e) return e;
-        e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, dtype, !reverse, nullptr, dlog_fgate,
-                                dvalue, query, key, loc_rem, nullptr, inner_ws, true);
+        e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, dtype, !reverse, nullptr, gates, dvalue,
+                                query, key, loc_rem, nullptr, inner_ws, true, gs);
         if (e) return e;
         loc2 = loc_rem;
     } else {
         e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, out_dtype, !reverse,
-                                lean ? nullptr : dleaving, dlog_fgate, dout, query, key, loc, dkey, inner_ws, true);
+                                lean ? nullptr : dleaving, gates, dout, query, key, loc, dkey, inner_ws, true, gs);
         if (e) return e;
     }
     // what enters segment p from the steps behind it: per piece, the gate of its first step (in the order of the

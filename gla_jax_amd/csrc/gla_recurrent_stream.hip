@@ -37,7 +37,7 @@ template <typename TO, int C, int D, bool STATE = false>
 __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_kernel(
     const void *__restrict__ h0, const float *__restrict__ g, const __bf16 *__restrict__ v,
     const __bf16 *__restrict__ k, const __bf16 *__restrict__ q, void *__restrict__ hT,
-    TO *__restrict__ out, int T_len, int H, int reverse, int hdt)
+    TO *__restrict__ out, int T_len, int H, int reverse, int hdt, int g_shift)
 {
     typedef __bf16 T;
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16;
@@ -98,15 +98,26 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
     f32x8 gN[KS];
     D8 qN[KS], kN[KS], vN[KS];
     bool validN;
-    int64_t rowN;
+    int64_t rowN, growN;
     auto fetch = [&](int n) {
         const int s = n * C + 16 * w + r;                      // logical step
         validN = s < T_len;
         const int sc = validN ? s : T_len - 1;
-        rowN = seq + (int64_t)(reverse ? T_len - 1 - sc : sc) * rowstride;
+        const int at = reverse ? T_len - 1 - sc : sc;
+        rowN = seq + (int64_t)at * rowstride;
+        growN = rowN;
+        if constexpr (STATE) {
+            // g_shift: a step takes the gate of the row g_shift rows further on in the array (the sequences of a
+            // launch lie one behind the other).  Where the array ends the nearest row stands in: that step is the
+            // first of its sequence, and its gate scales the zeros, or the initial state, it starts from.
+            int64_t gr = (int64_t)b * T_len + at + g_shift;
+            const int64_t last = (int64_t)gridDim.y * T_len - 1;
+            gr = gr < 0 ? 0 : (gr > last ? last : gr);
+            growN = (gr * H + h) * D;
+        }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            gN[ks] = ld8(g + rowN + 32 * ks + 8 * c);
+            gN[ks] = ld8(g + growN + 32 * ks + 8 * c);
             kN[ks] = ld8(k + rowN + 32 * ks + 8 * c);
             if constexpr (!STATE) qN[ks] = ld8(q + rowN + 32 * ks + 8 * c);
             else qN[ks] = kN[ks];                             // nothing uses the query side of a lean pass
@@ -118,7 +129,7 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
 #pragma unroll 1
     for (int n = 0; n < N; ++n) {
         const bool valid = validN;
-        const int64_t row = rowN;
+        const int64_t row = rowN, grow = growN;
         f32x4 accD = {0.f, 0.f, 0.f, 0.f};   // transposed scores of the own sub-block: [j = 4c+e][i = r]
         float qh[NV];                        // q * exp(l_i), walked down the earlier sub-blocks below
         {
@@ -140,7 +151,7 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
                 kf[ks] = kN[ks];
                 st8(Vn + wrow + 32 * ks, vN[ks]);
             }
-            subblock_forward<T, D, true, false, D == 64>(p, qf, kf, g + row, q + row, k + row, valid, rtab + w * D, Kh + wrow, true,
+            subblock_forward<T, D, true, false, D == 64>(p, qf, kf, g + grow, q + row, k + row, valid, rtab + w * D, Kh + wrow, true,
                                    Kl + wrow, r, c, accD, qh);
         }
         __syncthreads();                     // tiles of this block and the published state are in place
@@ -257,7 +268,7 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
 
 template <typename TO, int C, int D, bool STATE = false>
 static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, int hdt, const void *h0, const float *g,
-                      const void *v, const void *k, const void *q, void *hT, void *out)
+                      const void *v, const void *k, const void *q, void *hT, void *out, int g_shift = 0)
 {
     typedef __bf16 T;
     constexpr int LS = TileGeom<T, D>::kStride;
@@ -268,7 +279,7 @@ static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, int 
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, h0, g, (const T *)v, (const T *)k, (const T *)q, hT, (TO *)out,
-                       T_len, H, reverse, hdt);
+                       T_len, H, reverse, hdt, g_shift);
     return launch_status();
 }
 
@@ -283,10 +294,13 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
 }
 
 int launch_recurrent_stream_state(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, const void *h0,
-                                 const float *g, const void *v, const void *k, const void *q, void *hT)
+                                 const float *g, const void *v, const void *k, const void *q, void *hT, int g_shift)
 {
-    if (D == 64) return launch_one<__bf16, 128, 64, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, nullptr);
-    if (D == 128) return launch_one<__bf16, 64, 128, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, nullptr);
+    if (g_shift < -1 || g_shift > 1) return GLA_ERR_SHAPE;
+    if (D == 64)
+        return launch_one<__bf16, 128, 64, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, nullptr, g_shift);
+    if (D == 128)
+        return launch_one<__bf16, 64, 128, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, nullptr, g_shift);
     return GLA_ERR_UNSUPPORTED;
 }
 

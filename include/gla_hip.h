@@ -120,9 +120,9 @@ int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK,
  * recurrence is linear in the state, so one pass from zero states gives each segment's own contribution, a scan
  * over the segments the state that enters each (fp32, in the workspace), and a second pass the outputs; the
  * backward does the same for the states' cotangents first.  One workgroup walks one (batch, head) pair, so without
- * this a call with 8 pairs uses 8 of 256 compute units.  The backward keeps the gates moved by one row in
- * dlog_fgate and, where a pass writes an `out` nobody needs, that in dquery and dkey until it writes its results
- * there; an fp32 dout beside bf16 data (out_dtype != dtype) enters the cotangents' pass as two bf16 arrays, head and
+ * this a call with 8 pairs uses 8 of 256 compute units.  The backward uses its result arrays as scratch until it
+ * writes the results there (where the first passes are full kernels: the gates moved by one row in dlog_fgate, the
+ * passes' unused `out` in dquery and dkey); an fp32 dout beside bf16 data (out_dtype != dtype) enters the cotangents' pass as two bf16 arrays, head and
  * remainder, kept in dkey and dvalue (head dimensions 16 and 32 then run the backward on whole sequences).
  * The size functions return 0 where a workspace buys nothing; the entry points then ignore `workspace` (NULL is
  * fine) and behave exactly like the ones above.  Same results within the tolerance either way (segments: the
