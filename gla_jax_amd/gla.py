@@ -170,6 +170,9 @@ class _ChunkGLA(torch.autograd.Function):
         ctx.chunk_size = chunk_size
         ctx.hidden_dtype = h0.dtype
         ctx.mark_non_differentiable(states)
+        # no zeros for the cotangents nobody computed: `states` would get a 25 MB fill per step at B4 T4096 H6 D128;
+        # backward() makes the zeros that hidden_final and out need
+        ctx.set_materialize_grads(False)
 
     @staticmethod
     def backward(ctx, dhT, dout, dstates=None):
