@@ -399,7 +399,7 @@ def main():
         # the other BASELINE configs that fit one GPU, each with its own throughput and roofline fraction
         # (a few steps each; `--workload long|recurrent` gives the full line of one of them)
         other = {}
-        for name in ("long", "recurrent"):
+        for name in ("long", "recurrent", "recurrent_few"):
             k2, B2, T2, H2, D2, c2, s2 = WORKLOADS[name]
             n2 = max(5, min(args.steps, 10))
             r2 = bench_chunk(B2, T2, H2, D2, c2, s2, n2, 2, public=False) if k2 == "chunk" else \
