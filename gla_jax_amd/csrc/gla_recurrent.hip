@@ -610,17 +610,18 @@ static int recurrent_fwd_inner(void *stream, int64_t B, int64_t T, int64_t H, in
                                gla_dtype hidden_dtype, gla_dtype out_dtype, int reverse, const void *hidden_init,
                                const float *log_fgate, const void *value, const void *key, const void *query,
                                void *hidden_final, void *out, void *workspace, bool state_only = false,
-                               int g_shift = 0)
+                               int g_shift = 0, float *gate_sums = nullptr)
 {
     // state_only: the caller wants hidden_final alone and `out` is a buffer it will overwrite.  The matrix-core
     // kernels have a form without the output products (hidden_init may be null there: zeros); the other kernels
     // write the unused `out`.
     // g_shift (lean passes only): the gates are taken one row further on (+1) or back (-1), see the launcher.
     const bool lean = state_only && dtype == GLA_BF16;
-    if (g_shift && !(lean && DK >= 64)) return GLA_ERR_UNSUPPORTED;
+    // gate_sums (lean passes only): the pass also leaves the sum of every sequence's gates there, [B][H][DK].
+    if ((g_shift || gate_sums) && !(lean && DK >= 64)) return GLA_ERR_UNSUPPORTED;
     if (lean && (DK == 64 || DK == 128))
         return gla::launch_recurrent_stream_state((hipStream_t)stream, B, T, H, DK, reverse, hidden_dtype, hidden_init,
-                                                  log_fgate, value, key, query, hidden_final, g_shift);
+                                                  log_fgate, value, key, query, hidden_final, g_shift, gate_sums);
     if (DK != 256 || !workspace)
         return recurrent_fwd_run(stream, B, T, H, DK, DV, dtype, hidden_dtype, out_dtype, reverse, hidden_init,
                                  log_fgate, value, key, query, hidden_final, out);
@@ -640,7 +641,7 @@ static int recurrent_fwd_inner(void *stream, int64_t B, int64_t T, int64_t H, in
     // both in fp32 (the recurrent_gla_naive flavour of the 128-feature kernels)
     if (lean) {
         e = gla::launch_recurrent_stream_state(st, B, T, 2 * H, 128, reverse, hidden_dtype, hidden_init ? h0_same : nullptr,
-                                               log_fgate, value, key, query, hT_same, g_shift);
+                                               log_fgate, value, key, query, hT_same, g_shift, gate_sums);
         if (e) return e;
         e = gla::launch_recurrent_stream_state(st, B, T, 2 * H, 128, reverse, hidden_dtype,
                                                hidden_init ? h0_cross : nullptr, log_fgate, v_sw, key, query, hT_cross,
@@ -688,16 +689,17 @@ extern "C" int gla_recurrent_fwd_ws(void *stream, int64_t B, int64_t T, int64_t 
     void *inner_ws = DK == 256 ? ws + ts.fwd() : nullptr;
     const bool lean = gla::has_lean_pass(dtype, DK);
     const int64_t pieces = B * ts.S * ts.F;
-    int e = gla::launch_segment_gate_sums(st, B, ts.S * ts.F, ts.Lf, H, (int)DK, log_fgate, sums);
-    if (e) return e;
-    if (!lean) {            // (F = 1 then) the full kernels want an initial state: zeros
+    int e = 0;
+    if (!lean) {            // (F = 1 then) the full kernels want an initial state, zeros, and leave the gate sums to a kernel
+        e = gla::launch_segment_gate_sums(st, B, ts.S * ts.F, ts.Lf, H, (int)DK, log_fgate, sums);
+        if (e) return e;
         e = gla::launch_zero_fill(st, entering, ts.hid);
         if (e) return e;
     }
-    // every piece from a zero state: its own contribution to the state that leaves it (where this is a full pass, it
-    // writes an `out` that the pass below writes again)
+    // every piece from a zero state: its own contribution to the state that leaves it, and its gate sums (where this
+    // is a full pass, it writes an `out` that the pass below writes again)
     e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, lean ? nullptr : entering,
-                            log_fgate, value, key, query, loc, out, inner_ws, true);
+                            log_fgate, value, key, query, loc, out, inner_ws, true, 0, lean ? sums : nullptr);
     if (e) return e;
     e = gla::launch_segment_scan(st, B, ts.S, ts.F, ts.Lf, H, (int)DK, hidden_dtype, hidden_init, loc, nullptr, sums,
                                  nullptr, 0, reverse, entering, hidden_final);
@@ -836,16 +838,17 @@ extern "C" int gla_recurrent_bwd_ws(void *stream, int64_t B, int64_t T, int64_t 
     const bool lean = gla::has_lean_pass(dtype, DK);
     // 1. the states that enter the segments, as the forward formed them (where the pass is a full one, its `out` lands
     //    in dquery, which the backward proper overwrites)
-    int e = gla::launch_segment_gate_sums(st, B, ts.S * ts.F, ts.Lf, H, (int)DK, log_fgate, sums);
-    if (e) return e;
+    int e = 0;
     if (!lean) {
+        e = gla::launch_segment_gate_sums(st, B, ts.S * ts.F, ts.Lf, H, (int)DK, log_fgate, sums);
+        if (e) return e;
         e = gla::launch_zero_fill(st, entering, ts.hid);
         if (e) return e;
         e = gla::launch_zero_fill(st, dleaving, ts.hid);
         if (e) return e;
     }
     e = recurrent_fwd_inner(stream, pieces, ts.Lf, H, DK, DV, dtype, GLA_F32, out_dtype, reverse, lean ? nullptr : entering,
-                            log_fgate, value, key, query, loc, dquery, inner_ws, true);
+                            log_fgate, value, key, query, loc, dquery, inner_ws, true, 0, lean ? sums : nullptr);
     if (e) return e;
     e = gla::launch_segment_scan(st, B, ts.S, ts.F, ts.Lf, H, (int)DK, hidden_dtype, hidden_init, loc, nullptr, sums,
                                  nullptr, 0, reverse, entering, nullptr);

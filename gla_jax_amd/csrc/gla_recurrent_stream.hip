@@ -37,7 +37,7 @@ template <typename TO, int C, int D, bool STATE = false>
 __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_kernel(
     const void *__restrict__ h0, const float *__restrict__ g, const __bf16 *__restrict__ v,
     const __bf16 *__restrict__ k, const __bf16 *__restrict__ q, void *__restrict__ hT,
-    TO *__restrict__ out, int T_len, int H, int reverse, int hdt, int g_shift)
+    TO *__restrict__ out, int T_len, int H, int reverse, int hdt, int g_shift, float *__restrict__ gate_sums)
 {
     typedef __bf16 T;
     constexpr int NB = C / 16, KS = D / 32, NV = D / 4, NT = D / 16;
@@ -55,6 +55,7 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
     T *St = Kl + C * LS;                           // [D][LS]  state at the start of the block, [dv][dk]: bf16 head
     T *Sl = St + D * LS;                           // [D][LS]  ... and the bf16 of what the head leaves over
     float *rtab = reinterpret_cast<float *>(STATE ? St : Sl + D * LS);   // [NB][D] exp(tau_m)
+    float *gsum = rtab + NB * D;                   // [D] (STATE with gate_sums) the gates of the whole sequence, added up
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -93,6 +94,10 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
                 }
     };
     if constexpr (!STATE) publish_state();
+    if constexpr (STATE) {
+        if (gate_sums && threadIdx.x < D) gsum[threadIdx.x] = 0.f;
+        __syncthreads();                             // the other waves add to it before the loop's first barrier
+    }
 
     // inputs of the wave's 16 steps of a block, one block ahead
     f32x8 gN[KS];
@@ -153,6 +158,17 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
             }
             subblock_forward<T, D, true, false, D == 64>(p, qf, kf, g + grow, q + row, k + row, valid, rtab + w * D, Kh + wrow, true,
                                    Kl + wrow, r, c, accD, qh);
+            if constexpr (STATE) {
+                // the sequence's gate sums (what the scan over segments decays a state by): p now holds the sums
+                // over the sub-block's rows up to the lane's own, in powers of two, so its last row holds the
+                // sub-block's total (padded steps add zeros); one addition per feature, sub-block and block
+                if (gate_sums && r == 15) {
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) atomicAdd(gsum + 32 * ks + 8 * c + e, p[8 * ks + e]);
+                }
+            }
         }
         __syncthreads();                     // tiles of this block and the published state are in place
 
@@ -257,6 +273,10 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
         if constexpr (!STATE) publish_state();
     }
 
+    if constexpr (STATE) {
+        // (the loop's last barrier is behind every wave's additions)
+        if (gate_sums && threadIdx.x < D) gate_sums[bh * D + threadIdx.x] = gsum[threadIdx.x] * (1.f / kLog2e);
+    }
 #pragma unroll
     for (int i = 0; i < RT; ++i)
 #pragma unroll
@@ -268,18 +288,20 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
 
 template <typename TO, int C, int D, bool STATE = false>
 static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, int hdt, const void *h0, const float *g,
-                      const void *v, const void *k, const void *q, void *hT, void *out, int g_shift = 0)
+                      const void *v, const void *k, const void *q, void *hT, void *out, int g_shift = 0,
+                      float *gate_sums = nullptr)
 {
     typedef __bf16 T;
     constexpr int LS = TileGeom<T, D>::kStride;
     // (the lean form has no copy of the state in LDS; its table of decays moves up to where that copy would start)
-    const size_t lds = (size_t)(3 * C + (STATE ? 0 : 2 * D)) * LS * sizeof(T) + (size_t)(C / 16) * D * sizeof(float);
+    const size_t lds = (size_t)(3 * C + (STATE ? 0 : 2 * D)) * LS * sizeof(T) +
+                       (size_t)(C / 16 + (STATE ? 1 : 0)) * D * sizeof(float);
     auto kern = recurrent_stream_fwd_kernel<TO, C, D, STATE>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;
     dim3 grid(H, B), block(C * 4);
     hipLaunchKernelGGL(kern, grid, block, lds, st, h0, g, (const T *)v, (const T *)k, (const T *)q, hT, (TO *)out,
-                       T_len, H, reverse, hdt, g_shift);
+                       T_len, H, reverse, hdt, g_shift, gate_sums);
     return launch_status();
 }
 
@@ -294,13 +316,16 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
 }
 
 int launch_recurrent_stream_state(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, const void *h0,
-                                 const float *g, const void *v, const void *k, const void *q, void *hT, int g_shift)
+                                 const float *g, const void *v, const void *k, const void *q, void *hT, int g_shift,
+                                 float *gate_sums)
 {
-    if (g_shift < -1 || g_shift > 1) return GLA_ERR_SHAPE;
+    if (g_shift < -1 || g_shift > 1 || (g_shift && gate_sums)) return GLA_ERR_SHAPE;
     if (D == 64)
-        return launch_one<__bf16, 128, 64, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, nullptr, g_shift);
+        return launch_one<__bf16, 128, 64, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, nullptr, g_shift,
+                                                 gate_sums);
     if (D == 128)
-        return launch_one<__bf16, 64, 128, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, nullptr, g_shift);
+        return launch_one<__bf16, 64, 128, true>(st, B, T_len, H, reverse, hdt, h0, g, v, k, q, hT, nullptr, g_shift,
+                                                 gate_sums);
     return GLA_ERR_UNSUPPORTED;
 }
 

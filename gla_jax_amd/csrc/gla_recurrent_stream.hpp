@@ -16,9 +16,10 @@ int launch_recurrent_stream_fwd(hipStream_t st, int B, int T_len, int H, int D, 
 // h0 may be null: the state starts from zeros.  g_shift = +1 or -1: every step takes the gate of the next (previous)
 // row of the array instead of its own (the recurrence of the state's cotangent, where the decay between two steps
 // belongs to the later one); the first step of a sequence, whose gate scales the initial state, may get any row's.
+// gate_sums (may be null; not with g_shift): [B][H][D] floats, the sum of every sequence's gates.
 int launch_recurrent_stream_state(hipStream_t st, int B, int T_len, int H, int D, int reverse, int hdt, const void *h0,
                                  const float *g, const void *v, const void *k, const void *q, void *hT,
-                                 int g_shift = 0);
+                                 int g_shift = 0, float *gate_sums = nullptr);
 
 // Sweep 1 of the backward: dq, and q*dq in fp32 into `qdq` (the last step's carries sum_v dhT * (final state)
 // on top).  dout_f32 != 0: `dout` is float (the recurrent_gla_naive flavour), else bf16.  wide != 0 (head dimension
