@@ -10,8 +10,10 @@
 // cotangent of the state at every segment's end as well: it obeys the same kind of recurrence against time, with
 // query in the place of key, dout in the place of value and the decays moved by one step (the decay between
 // two steps belongs to the later one).  States cross segments in fp32.
-// This file holds the small kernels around those passes: the segments' gate sums, the gates moved by one row,
-// the scan over segments, a zero fill.
+// This file holds the small kernels around those passes: the scan over segments, a float array as two bf16 arrays
+// (an fp32 dout beside bf16 data) and, for the cases whose first pass is a full kernel (fp32 data, head dimensions 16
+// and 32; the lean kernel of the others does these itself), the segments' gate sums, the gates moved by one row and
+// a zero fill.
 #include "gla_timesplit.hpp"
 
 namespace gla {
