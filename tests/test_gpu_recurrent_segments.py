@@ -138,3 +138,69 @@ def test_segmented_recurrent_gla_naive_flavour(B, T, H, D, reverse):
     exp = O.recurrent_gla_naive_grad(h0, g, v, k, q, dhT, dout, reverse=reverse)
     assert_plain("out", to_np(out), exp[6], 1e-4)
     print(fmt_log(check_recurrent_outputs(dtype, exp, hT, out, grads, out_fp32=True)))
+
+
+def test_random_shapes_in_segments_agree_with_whole_sequences():
+    """A fixed-seed draw of shapes that run in segments (both element types, fp32 states beside bf16 data, the
+    recurrent_gla_naive flavour, every head dimension, lengths that are odd multiples of 256, both directions,
+    scattered resets), each through the entry points with a workspace and through those without.  The case is
+    printed before it runs."""
+    from gla_jax_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(20240611)
+    p = lambda t: t.data_ptr()
+    done = 0
+    for it in range(40):
+        dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float32
+        dt = _lib.GLA_BF16 if dtype == torch.bfloat16 else _lib.GLA_F32
+        hd = torch.float32 if rng.random() < 0.3 else dtype
+        hdt = _lib.GLA_BF16 if hd == torch.bfloat16 else _lib.GLA_F32
+        D = int(rng.choice([16, 32, 64, 64, 128, 128, 256]))
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        T = int(rng.choice([512, 1024, 1280, 1536, 2048, 2560, 3072]))
+        if D == 256 or dtype == torch.float32:
+            T = min(T, 1536)                       # the whole-sequence vector kernels are slow
+        rev = int(rng.integers(0, 2))
+        naive = dtype == torch.bfloat16 and rng.random() < 0.25
+        odt, otype = (_lib.GLA_F32, torch.float32) if naive else (dt, dtype)
+        shift = float(rng.choice([0.0, 1.0, 3.0, 5.0]))
+        nf, nb = _sizes(B, T, H, D, dtype)
+        print(f"case {it}: {dtype} states {hd} fp32-out {naive} B{B} T{T} H{H} D{D} reverse {rev} shift {shift} "
+              f"workspace {nf} {nb}", flush=True)
+        if nf == 0:
+            continue
+        gen = torch.Generator(device="cuda").manual_seed(1000 + it)
+        rand = lambda *s, t=dtype: torch.randn(*s, device="cuda", generator=gen).to(t)
+        g = torch.nn.functional.logsigmoid(shift + rand(B, T, H, D, t=torch.float32))
+        if rng.random() < 0.5:
+            g[:, torch.as_tensor(rng.integers(0, T, size=5), device="cuda")] = float(rng.choice([-200.0, -30.0]))
+        h0, dhT = rand(B, H, D, D, t=hd), rand(B, H, D, D, t=hd)
+        v, k, q, dout = rand(B, T, H, D), rand(B, T, H, D), rand(B, T, H, D), rand(B, T, H, D, t=otype)
+        outs = lambda: [torch.empty_like(h0), torch.empty_like(dout), torch.empty_like(h0), torch.empty_like(g),
+                        torch.empty_like(v), torch.empty_like(k), torch.empty_like(q)]
+        ws_f = torch.full((nf,), 77, dtype=torch.uint8, device="cuda")
+        ws_b = torch.full((nb,), 77, dtype=torch.uint8, device="cuda")
+        st = torch.cuda.current_stream().cuda_stream
+        whole, seg = outs(), outs()
+        hT, out, dh0, dg, dv, dk, dq = whole
+        _lib.check("gla_recurrent_fwd", lib.gla_recurrent_fwd(st, B, T, H, D, D, dt, hdt, odt, rev, p(h0), p(g), p(v), p(k),
+                                                              p(q), p(hT), p(out)))
+        _lib.check("gla_recurrent_bwd", lib.gla_recurrent_bwd(st, B, T, H, D, D, dt, hdt, odt, rev, p(h0), p(g), p(v), p(k),
+                                                              p(q), p(hT), p(dhT), p(dout), p(dh0), p(dg), p(dv), p(dk),
+                                                              p(dq)))
+        hT, out, dh0, dg, dv, dk, dq = seg
+        _lib.check("gla_recurrent_fwd_ws", lib.gla_recurrent_fwd_ws(st, B, T, H, D, D, dt, hdt, odt, rev, p(h0), p(g), p(v),
+                                                                    p(k), p(q), p(hT), p(out), p(ws_f), nf))
+        _lib.check("gla_recurrent_bwd_ws", lib.gla_recurrent_bwd_ws(st, B, T, H, D, D, dt, hdt, odt, rev, p(h0), p(g), p(v),
+                                                                    p(k), p(q), p(hT), p(dhT), p(dout), p(dh0), p(dg), p(dv),
+                                                                    p(dk), p(dq), p(ws_b), nb))
+        torch.cuda.synchronize()
+        for name, a, b in zip(("hidden_final", "out", "dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), whole, seg):
+            x, y = a.double(), b.double()
+            worst = float((x - y).abs().max()) / float(x.pow(2).mean().sqrt())
+            # a float result: the order of fp32 sums (d(log_fgate) of bf16 data: two forms of the carried sum, 1e-4
+            # each); a bf16 result: a rounding step of a value of up to 16 RMS
+            bound = 2e-3 if a.dtype == torch.float32 else 6.3e-2
+            assert worst <= bound, f"case {it} {name}: {worst:.3e}"
+        done += 1
+    assert done >= 25
