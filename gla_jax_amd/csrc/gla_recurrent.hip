@@ -553,8 +553,13 @@ struct TimeSplit {
     TimeSplit(int64_t B, int64_t T, int64_t H, int64_t DK, int dtype)
     {
         const int64_t seqs = B * H * (DK == 256 ? 2 : 1);    // head dimension 256 runs as 2H heads of 128
-        while (seqs * S * 2 <= kComputeUnits && T % (S * 2) == 0 && T / (S * 2) >= kMinSegment && B * S * 2 <= 65535)
-            S *= 2;
+        // the most segments that divide T into pieces of kMinSegment steps or more without asking for more
+        // workgroups than there are compute units
+        for (int64_t s = kComputeUnits / (seqs > 0 ? seqs : 1); s > 1; --s)
+            if (T % s == 0 && T / s >= kMinSegment && B * s <= 65535) {
+                S = s;
+                break;
+            }
         // Two segments mean two passes over half the steps each: that pays only where the first pass is the lean one
         // (bf16 data) and the kernels are heavy (128 features: 1.47 -> 1.32 ms at B16 T2048 H8; 64 features:
         // 0.43 -> 0.45 ms).  From four segments on it pays everywhere.
