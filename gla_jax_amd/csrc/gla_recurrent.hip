@@ -536,8 +536,8 @@ extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, 
 }
 
 // ---- a sequence as S segments side by side (gla_timesplit.hip) -------------------------------------------------
-// With fewer (batch, head) pairs than a quarter of the GPU's compute units, a call with a workspace runs every
-// sequence as S segments at once: one pass from zero states for the segments' own contributions, a scan over the
+// With few (batch, head) pairs (at most a quarter of the GPU's compute units; half of them for bf16 data at 128
+// features and more), a call with a workspace runs every sequence as S segments at once: one pass from zero states for the segments' own contributions, a scan over the
 // segments, and the real pass with the states that enter each segment (fp32); the backward does the same for
 // the states' cotangents.  The segments are batch entries of the same kernels: [B,T,H,D] is [B*S,T/S,H,D].
 namespace gla {
