@@ -81,17 +81,32 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
             if (h0) load_hidden<4>(h0, hdt, bh * D * D + (int64_t)(16 * (nt0 + nt) + r) * D + 16 * (wv + i * NDV) + 4 * c, t4);
             S[i][nt] = f32x4{t4[0], t4[1], t4[2], t4[3]};
         }
+    // A lane's four values of a tile lie in four rows of the [dv][dk] copy.  The four lanes of a quad exchange them
+    // (a 4 x 4 transpose in two steps across lanes 1 and 2 apart), after which lane 4a + j holds the key features
+    // 4a..4a+3 of row 4c + j: one 8-byte store per tile and precision instead of four 2-byte ones.
     auto publish_state = [&]() {
+        const int j = r & 3;
 #pragma unroll
         for (int i = 0; i < RT; ++i)
 #pragma unroll
-            for (int nt = 0; nt < NTW; ++nt)
+            for (int nt = 0; nt < NTW; ++nt) {
+                f32x4 x = S[i][nt], y;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const T hi = (T)S[i][nt][e];
-                    St[(16 * (wv + i * NDV) + 4 * c + e) * LS + 16 * (nt0 + nt) + r] = hi;
-                    Sl[(16 * (wv + i * NDV) + 4 * c + e) * LS + 16 * (nt0 + nt) + r] = (T)(S[i][nt][e] - (float)hi);
+                    const float other = dpp_f32<kDppQuadXor1>(x[e ^ 1]);
+                    y[e] = ((j ^ e) & 1) ? other : x[e];
                 }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float other = dpp_f32<kDppQuadXor2>(y[e ^ 2]);
+                    x[e] = ((j ^ e) & 2) ? other : y[e];
+                }
+                T4 hi, lo;
+                split4<T>(x, hi, lo);
+                const int off = (16 * (wv + i * NDV) + 4 * c + j) * LS + 16 * (nt0 + nt) + (r & 12);
+                *reinterpret_cast<T4 *>(St + off) = hi;
+                *reinterpret_cast<T4 *>(Sl + off) = lo;
+            }
     };
     if constexpr (!STATE) publish_state();
     if constexpr (STATE) {
