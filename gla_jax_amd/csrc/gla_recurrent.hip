@@ -536,8 +536,8 @@ extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, 
 }
 
 // ---- a sequence as S segments side by side (gla_timesplit.hip) -------------------------------------------------
-// With few (batch, head) pairs (at most a quarter of the GPU's compute units; half of them for bf16 data at 128
-// features and more), a call with a workspace runs every sequence as S segments at once: one pass from zero states for the segments' own contributions, a scan over the
+// With few (batch, head) pairs (at most half of the GPU's compute units for bf16 data at 64 features and more, a
+// quarter otherwise), a call with a workspace runs every sequence as S segments at once: one pass from zero states for the segments' own contributions, a scan over the
 // segments, and the real pass with the states that enter each segment (fp32); the backward does the same for
 // the states' cotangents.  The segments are batch entries of the same kernels: [B,T,H,D] is [B*S,T/S,H,D].
 namespace gla {
@@ -560,11 +560,11 @@ struct TimeSplit {
                 S = s;
                 break;
             }
-        // Two segments mean two passes over half the steps each: that pays only where the first pass is the lean one
-        // (bf16 data) and the kernels are heavy (128 features: 1.47 -> 1.32 ms at B16 T2048 H8; 64 features:
-        // 0.43 -> 0.45 ms).  From four segments on it pays everywhere.
+        // Two segments mean two passes over half the steps each: that pays where the first pass is the lean one (bf16
+        // data at 64 features and more: B16 T2048 H8 1.47 -> 1.08 ms at 128 features, 0.44 -> 0.39 ms at 64); where it
+        // is a full kernel, from four segments on.
         const bool heavy = dtype == GLA_BF16 && DK >= 128;
-        if (S < (heavy ? 2 : 4)) S = 1;
+        if (S < (has_lean_pass(dtype, DK) ? 2 : 4)) S = 1;
         L = T / S;
         // The lean kernel of 128 features fits a compute unit twice (256 registers, 52 KB of LDS) where the full
         // kernels fit once: its passes take every segment in two pieces (512 workgroups: 100 -> 70 us at 1024 steps

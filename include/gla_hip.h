@@ -115,8 +115,9 @@ int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK,
  * matrix cores for bf16 data, with the passes' results kept in fp32 in the workspace and rounded once.  Without a
  * workspace (the two entry points above) head dimension 256 runs on per-timestep vector kernels, an order of
  * magnitude slower.
- * (2) With few sequences (B*H, at head dimension 256 2*B*H, at most a quarter of the GPU's 256 compute units) and
- * T a multiple of S >= 4 segments of at least 256 steps, every sequence runs as S segments side by side: the
+ * (2) With few sequences (B*H, at head dimension 256 2*B*H, at most half of the GPU's 256 compute units for bf16
+ * data at head dimensions 64 and more, a quarter otherwise) and T a multiple of S segments of at least 256 steps,
+ * every sequence runs as S segments side by side: the
  * recurrence is linear in the state, so one pass from zero states gives each segment's own contribution, a scan
  * over the segments the state that enters each (fp32, in the workspace), and a second pass the outputs; the
  * backward does the same for the states' cotangents first.  One workgroup walks one (batch, head) pair, so without

@@ -87,7 +87,7 @@ def test_chunk_plan_and_sizes():
     assert lib.gla_chunk_states_bytes(B, T, H, 512, 512, 128, _lib.GLA_BF16) == 0
     # recurrent_gla: a workspace at head dimension 256 (both passes' results in fp32 and the exchanged rows) and, at
     # every head dimension, where the sequences are few enough to run as S >= 4 segments of >= 256 steps side by
-    # side (B*H*S <= 256 workgroups; S = 2 already for bf16 data at head dimensions 128 and 256): the segments'
+    # side (B*H*S <= 256 workgroups; S = 2 already for bf16 data at head dimensions 64 and more): the segments'
     # states in fp32, twice (backward: four times), and their gate sums
     r256 = lambda x: (x + 255) & ~255
     for D in (16, 32, 64, 128):
@@ -98,7 +98,7 @@ def test_chunk_plan_and_sizes():
         # contributions and the gate sums count twice)
         F = 2 if D == 128 else 1
         two = lib.gla_recurrent_fwd_workspace_bytes(16, 2048, 8, D, D, _lib.GLA_BF16)           # 128 sequences: S = 2
-        assert two == (3 * r256(16 * 2 * 8 * D * D * 4) + r256(16 * 4 * 8 * D * 4) if D == 128 else 0)
+        assert two == ((1 + F) * r256(16 * 2 * 8 * D * D * 4) + r256(16 * 2 * F * 8 * D * 4) if D >= 64 else 0)
         S = 8                                                                                   # 24 sequences of 4096 steps
         hid, sums = r256(B * S * H * D * D * 4), r256(B * S * H * D * 4)
         assert lib.gla_recurrent_fwd_workspace_bytes(B, T, H, D, D, _lib.GLA_BF16) == (1 + F) * hid + F * sums

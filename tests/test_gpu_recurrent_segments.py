@@ -24,7 +24,9 @@ CASES = [
     (torch.bfloat16, 1, 1024, 1, 256, True, 3.0),
     (torch.bfloat16, 1, 1200, 2, 64, False, 3.0),       # 4 segments of 300 steps: not a multiple of the kernels' blocks
     (torch.bfloat16, 1, 1280, 3, 64, True, 3.0),        # 5 segments of 256 steps
-    (torch.bfloat16, 1, 512, 2, 128, False, 3.0),       # two segments (bf16 at head dimensions 128 and 256 only)
+    (torch.bfloat16, 1, 512, 2, 128, False, 3.0),       # two segments (bf16 at head dimensions 64 and more only)
+    (torch.bfloat16, 2, 512, 1, 64, True, 3.0),
+    (torch.bfloat16, 1, 768, 2, 64, False, 1.0),        # three
     (torch.bfloat16, 2, 512, 1, 128, True, 1.0),
     (torch.bfloat16, 1, 512, 1, 256, False, 3.0),
     (torch.bfloat16, 1, 2048, 64, 128, False, 3.0),     # 4 segments of 512 steps, the lean passes in pieces of 256
