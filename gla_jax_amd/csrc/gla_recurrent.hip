@@ -542,7 +542,9 @@ extern "C" int gla_recurrent_fwd(void *stream, int64_t B, int64_t T, int64_t H, 
 // the states' cotangents.  The segments are batch entries of the same kernels: [B,T,H,D] is [B*S,T/S,H,D].
 namespace gla {
 constexpr int64_t kComputeUnits = 256;       // MI355X
-constexpr int64_t kMinSegment = 256;         // steps: below this the extra pass costs more than the idle units
+constexpr int64_t kMinSegment = 128;         // steps: one or two iterations of the kernels (with 256 the small shapes left
+                                             // compute units idle: B1 T2048 H4 D128 0.31 -> 0.20 ms, B1 T1024 H8 D64 0.11 -> 0.08)
+constexpr int64_t kMinLeanPiece = 256;       // steps of a piece where the lean passes take a segment in two
 // bf16 data at head dimensions 64, 128 (and 256 as two passes of 128): the forward kernel has a form that leaves out
 // everything but the state
 static inline bool has_lean_pass(int dtype, int64_t DK) { return dtype == GLA_BF16 && DK >= 64; }
@@ -570,7 +572,7 @@ struct TimeSplit {
         // kernels fit once: its passes take every segment in two pieces (512 workgroups: 100 -> 70 us at 1024 steps
         // per segment), and the scan puts the pieces together.  Pieces of 128 steps are two iterations of the kernel
         // and lose what the second workgroup gains.
-        if (S > 1 && heavy && L % 2 == 0 && L / 2 >= kMinSegment && B * S * 2 <= 65535) F = 2;
+        if (S > 1 && heavy && L % 2 == 0 && L / 2 >= kMinLeanPiece && B * S * 2 <= 65535) F = 2;
         Lf = L / F;
         hid = SplitSizes::round_up256((size_t)B * S * H * DK * DK * 4);
         hidf = SplitSizes::round_up256((size_t)B * S * F * H * DK * DK * 4);

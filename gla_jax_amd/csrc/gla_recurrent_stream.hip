@@ -55,7 +55,7 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
     T *St = Kl + C * LS;                           // [D][LS]  state at the start of the block, [dv][dk]: bf16 head
     T *Sl = St + D * LS;                           // [D][LS]  ... and the bf16 of what the head leaves over
     float *rtab = reinterpret_cast<float *>(STATE ? St : Sl + D * LS);   // [NB][D] exp(tau_m)
-    float *gsum = rtab + NB * D;                   // [D] (STATE with gate_sums) the gates of the whole sequence, added up
+    float *gsum = rtab + NB * D;                   // [NB][D] (STATE with gate_sums) every wave's share of the sequence's gate sums
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -110,8 +110,9 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
     };
     if constexpr (!STATE) publish_state();
     if constexpr (STATE) {
-        if (gate_sums && threadIdx.x < D) gsum[threadIdx.x] = 0.f;
-        __syncthreads();                             // the other waves add to it before the loop's first barrier
+        if (gate_sums)
+            for (int d = threadIdx.x; d < NB * D; d += C * 4) gsum[d] = 0.f;
+        __syncthreads();                             // a wave adds to its row before the loop's first barrier
     }
 
     // inputs of the wave's 16 steps of a block, one block ahead
@@ -176,12 +177,16 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
             if constexpr (STATE) {
                 // the sequence's gate sums (what the scan over segments decays a state by): p now holds the sums
                 // over the sub-block's rows up to the lane's own, in powers of two, so its last row holds the
-                // sub-block's total (padded steps add zeros); one addition per feature, sub-block and block
+                // sub-block's total (padded steps add zeros).  Every wave keeps a row of its own, added up in wave
+                // order at the end: the same bits whenever the same call runs again
                 if (gate_sums && r == 15) {
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks)
+                    for (int ks = 0; ks < KS; ++ks) {
+                        f32x8 t = ld8(gsum + w * D + 32 * ks + 8 * c);
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) atomicAdd(gsum + 32 * ks + 8 * c + e, p[8 * ks + e]);
+                        for (int e = 0; e < 8; ++e) t.v[e] += p[8 * ks + e];
+                        st8(gsum + w * D + 32 * ks + 8 * c, t);
+                    }
                 }
             }
         }
@@ -290,7 +295,12 @@ __global__ __launch_bounds__(C * 4, STATE ? 2 : 1) void recurrent_stream_fwd_ker
 
     if constexpr (STATE) {
         // (the loop's last barrier is behind every wave's additions)
-        if (gate_sums && threadIdx.x < D) gate_sums[bh * D + threadIdx.x] = gsum[threadIdx.x] * (1.f / kLog2e);
+        if (gate_sums && threadIdx.x < D) {
+            float t = 0.f;
+#pragma unroll
+            for (int m = 0; m < NB; ++m) t += gsum[m * D + threadIdx.x];
+            gate_sums[bh * D + threadIdx.x] = t * (1.f / kLog2e);
+        }
     }
 #pragma unroll
     for (int i = 0; i < RT; ++i)
@@ -310,7 +320,7 @@ static int launch_one(hipStream_t st, int B, int T_len, int H, int reverse, int 
     constexpr int LS = TileGeom<T, D>::kStride;
     // (the lean form has no copy of the state in LDS; its table of decays moves up to where that copy would start)
     const size_t lds = (size_t)(3 * C + (STATE ? 0 : 2 * D)) * LS * sizeof(T) +
-                       (size_t)(C / 16 + (STATE ? 1 : 0)) * D * sizeof(float);
+                       (size_t)(C / 16) * (STATE ? 2 : 1) * D * sizeof(float);
     auto kern = recurrent_stream_fwd_kernel<TO, C, D, STATE>;
     static LdsGrant grant;
     if (int e = allow_lds(grant, (const void *)kern, lds)) return e;

@@ -87,18 +87,37 @@ __global__ __launch_bounds__(256) void segment_scan_kernel(const void *__restric
     const int P = S * F;
     float x[4];
     load_hidden<4>(init, hdt, e, x);
-    for (int j = 0; j < P; ++j) {
-        const int pf = descending ? P - 1 - j : j;      // the piece, in the order the recurrence meets them
-        const int64_t piece = b * P + pf;
-        const int64_t o = (piece * H + h) * dd + in_state;
-        f32x4 l = *reinterpret_cast<const f32x4 *>(loc + o);
-        if (loc2) l += *reinterpret_cast<const f32x4 *>(loc2 + o);
-        if (j % F == 0)
-            *reinterpret_cast<f32x4 *>(entering + (((b * S + pf / F) * H + h) * dd + in_state)) = f32x4{x[0], x[1], x[2], x[3]};
-        const float a = expf(sums[(piece * H + h) * (int64_t)D + dk]);
-        const float w = g ? expf(g[((piece * Lf + edge_row) * H + h) * (int64_t)D + dk]) : 1.f;
+    // Only x ties one piece to the next; what a piece reads does not depend on it.  Eight pieces' reads are issued
+    // before the first of them is used: with few sequences there are few threads here and many pieces, and one
+    // piece per memory round trip made this kernel the longest of a call (36 us at 64 pieces of B1 T8192 H2 D64).
+    constexpr int kAhead = 8;
+    for (int j0 = 0; j0 < P; j0 += kAhead) {
+        f32x4 l[kAhead];
+        float a[kAhead], w[kAhead];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) x[c] = a * x[c] + w * l[c];
+        for (int u = 0; u < kAhead; ++u) {
+            const int j = j0 + u < P ? j0 + u : P - 1;      // (past the end: the last piece again, not used)
+            const int pf = descending ? P - 1 - j : j;      // the piece, in the order the recurrence meets them
+            const int64_t piece = b * P + pf;
+            const int64_t o = (piece * H + h) * dd + in_state;
+            l[u] = *reinterpret_cast<const f32x4 *>(loc + o);
+            if (loc2) l[u] += *reinterpret_cast<const f32x4 *>(loc2 + o);
+            a[u] = sums[(piece * H + h) * (int64_t)D + dk];
+            w[u] = g ? g[((piece * Lf + edge_row) * H + h) * (int64_t)D + dk] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int j = j0 + u;
+            if (j < P) {
+                const int pf = descending ? P - 1 - j : j;
+                if (j % F == 0)
+                    *reinterpret_cast<f32x4 *>(entering + (((b * S + pf / F) * H + h) * dd + in_state)) =
+                        f32x4{x[0], x[1], x[2], x[3]};
+                const float ea = expf(a[u]), ew = expf(w[u]);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) x[c] = ea * x[c] + ew * l[u][c];
+            }
+        }
     }
     if (final) store_hidden<4>(final, hdt, e, x);
 }

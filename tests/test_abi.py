@@ -86,14 +86,14 @@ def test_chunk_plan_and_sizes():
         sub + 16 * rows + hid + 12 * 256)
     assert lib.gla_chunk_states_bytes(B, T, H, 512, 512, 128, _lib.GLA_BF16) == 0
     # recurrent_gla: a workspace at head dimension 256 (both passes' results in fp32 and the exchanged rows) and, at
-    # every head dimension, where the sequences are few enough to run as S >= 4 segments of >= 256 steps side by
+    # every head dimension, where the sequences are few enough to run as S >= 4 segments of >= 128 steps side by
     # side (B*H*S <= 256 workgroups; S = 2 already for bf16 data at head dimensions 64 and more): the segments'
     # states in fp32, twice (backward: four times), and their gate sums
     r256 = lambda x: (x + 255) & ~255
     for D in (16, 32, 64, 128):
         assert lib.gla_recurrent_fwd_workspace_bytes(16, 2048, 16, D, D, _lib.GLA_BF16) == 0    # 256 sequences
         assert lib.gla_recurrent_bwd_workspace_bytes(16, 2048, 8, D, D, _lib.GLA_F32) == 0      # 128: S would be 2
-        assert lib.gla_recurrent_fwd_workspace_bytes(1, 500, 2, D, D, _lib.GLA_BF16) == 0       # segments below 256 steps
+        assert lib.gla_recurrent_fwd_workspace_bytes(1, 200, 2, D, D, _lib.GLA_BF16) == 0       # segments below 128 steps
         # (bf16 data at head dimension 128: the first pass takes every segment in F = 2 pieces, so its array of
         # contributions and the gate sums count twice)
         F = 2 if D == 128 else 1

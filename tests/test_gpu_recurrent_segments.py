@@ -22,13 +22,13 @@ CASES = [
     (torch.bfloat16, 1, 1024, 3, 16, False, 3.0),
     (torch.bfloat16, 2, 1024, 1, 256, False, 3.0),
     (torch.bfloat16, 1, 1024, 1, 256, True, 3.0),
-    (torch.bfloat16, 1, 1200, 2, 64, False, 3.0),       # 4 segments of 300 steps: not a multiple of the kernels' blocks
-    (torch.bfloat16, 1, 1280, 3, 64, True, 3.0),        # 5 segments of 256 steps
-    (torch.bfloat16, 1, 512, 2, 128, False, 3.0),       # two segments (bf16 at head dimensions 64 and more only)
-    (torch.bfloat16, 2, 512, 1, 64, True, 3.0),
-    (torch.bfloat16, 1, 768, 2, 64, False, 1.0),        # three
-    (torch.bfloat16, 2, 512, 1, 128, True, 1.0),
-    (torch.bfloat16, 1, 512, 1, 256, False, 3.0),
+    (torch.bfloat16, 1, 1200, 2, 64, False, 3.0),       # 8 segments of 150 steps: not a multiple of the kernels' blocks
+    (torch.bfloat16, 1, 1280, 3, 64, True, 3.0),        # 10 segments of 128 steps
+    (torch.bfloat16, 1, 256, 2, 128, False, 3.0),       # two segments (bf16 at head dimensions 64 and more only)
+    (torch.bfloat16, 2, 256, 1, 128, True, 1.0),
+    (torch.bfloat16, 1, 256, 1, 256, False, 3.0),
+    (torch.bfloat16, 2, 256, 1, 64, True, 3.0),
+    (torch.bfloat16, 1, 384, 2, 64, False, 1.0),        # three
     (torch.bfloat16, 1, 2048, 64, 128, False, 3.0),     # 4 segments of 512 steps, the lean passes in pieces of 256
     (torch.bfloat16, 2, 2048, 16, 256, True, 3.0),
 ]
@@ -69,6 +69,7 @@ def test_segmented_recurrent_gla_matches_oracle(dtype, B, T, H, D, reverse, shif
 
 @pytest.mark.parametrize("dtype,B,T,H,D,reverse", [(torch.bfloat16, 1, 1024, 2, 64, False),
                                                     (torch.bfloat16, 1, 1024, 1, 128, True),
+                                                    (torch.bfloat16, 2, 4096, 8, 64, False),
                                                     (torch.float32, 1, 1024, 2, 32, False)])
 def test_segments_agree_with_whole_sequences(dtype, B, T, H, D, reverse):
     """The same call through gla_recurrent_fwd / _bwd (no workspace: whole sequences) and through the _ws entry
@@ -101,7 +102,19 @@ def test_segments_agree_with_whole_sequences(dtype, B, T, H, D, reverse):
     _lib.check("gla_recurrent_bwd_ws", lib.gla_recurrent_bwd_ws(st, B, T, H, D, D, dt, dt, dt, rv, p(h0), p(g), p(v), p(k),
                                                                 p(q), p(hT), p(dhT), p(dout), p(dh0), p(dg), p(dv), p(dk),
                                                                 p(dq), p(ws_b), nb))
+    # the same call again: the same bits (no result depends on the order in which workgroups or waves finish)
+    again = outs()
+    hT, out, dh0, dg, dv, dk, dq = again
+    ws_f.fill_(1)
+    ws_b.fill_(2)
+    _lib.check("gla_recurrent_fwd_ws", lib.gla_recurrent_fwd_ws(st, B, T, H, D, D, dt, dt, dt, rv, p(h0), p(g), p(v), p(k),
+                                                                p(q), p(hT), p(out), p(ws_f), nf))
+    _lib.check("gla_recurrent_bwd_ws", lib.gla_recurrent_bwd_ws(st, B, T, H, D, D, dt, dt, dt, rv, p(h0), p(g), p(v), p(k),
+                                                                p(q), p(hT), p(dhT), p(dout), p(dh0), p(dg), p(dv), p(dk),
+                                                                p(dq), p(ws_b), nb))
     torch.cuda.synchronize()
+    for name, a, b in zip(("hidden_final", "out", "dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), seg, again):
+        assert torch.equal(a, b), f"{name} differs between two runs of the same call"
     for name, a, b in zip(("hidden_final", "out", "dhidden_init", "dlog_fgate", "dvalue", "dkey", "dquery"), whole, seg):
         a, b = to_np(a), to_np(b)
         rms = float(np.sqrt(np.mean(a ** 2)))
