@@ -562,6 +562,12 @@ struct TimeSplit {
                 S = s;
                 break;
             }
+        // At 128 features an iteration of the kernels is 64 steps, and segments of one iteration still pay while they
+        // leave half of the compute units idle or more (B1 T2048 H4 D128 0.20 -> 0.17 ms); beyond that a segment's
+        // own state, read and written once per pass, outweighs its 64 rows (B1 T8192 H2 D128 0.27 -> 0.29 ms).
+        if (DK >= 128 && S > 1 && seqs * S * 2 <= kComputeUnits / 2 && (T / S) % 2 == 0 && T / S / 2 >= 64 &&
+            B * S * 2 <= 65535)
+            S *= 2;
         // Two segments mean two passes over half the steps each: that pays where the first pass is the lean one (bf16
         // data at 64 features and more: B16 T2048 H8 1.47 -> 1.08 ms at 128 features, 0.44 -> 0.39 ms at 64); where it
         // is a full kernel, from four segments on.
