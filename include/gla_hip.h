@@ -116,9 +116,9 @@ int gla_recurrent_bwd(void *stream, int64_t B, int64_t T, int64_t H, int64_t DK,
  * workspace (the two entry points above) head dimension 256 runs on per-timestep vector kernels, an order of
  * magnitude slower.
  * (2) With few sequences (B*H, at head dimension 256 2*B*H, at most half of the GPU's 256 compute units for bf16
- * data at head dimensions 64 and more, a quarter otherwise) and T a multiple of S segments of at least 128 steps (64 at head dimensions 128 and 256 while few workgroups result),
- * every sequence runs as S segments side by side: the
- * recurrence is linear in the state, so one pass from zero states gives each segment's own contribution, a scan
+ * data at head dimensions 64 and more, a quarter otherwise) and T a multiple of S segments of at least 128 steps
+ * (64 at head dimensions 128 and 256 while few workgroups result), every sequence runs as S segments side by side:
+ * the recurrence is linear in the state, so one pass from zero states gives each segment's own contribution, a scan
  * over the segments the state that enters each (fp32, in the workspace), and a second pass the outputs; the
  * backward does the same for the states' cotangents first.  One workgroup walks one (batch, head) pair, so without
  * this a call with 8 pairs uses 8 of 256 compute units.  The backward uses its result arrays as scratch until it
